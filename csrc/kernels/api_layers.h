@@ -1,0 +1,138 @@
+// Host-visible API of the layer-mechanism kernels that serve configuration-driven designs (layers listed in a
+// checkpoint's config.json): the general row-major GEMM, the one-number RMS norm on a sublayer's output, latent
+// (compressed-KV) attention with a sliding window, the gated linear recurrence with its short convolution, and the
+// routed mixture of experts.  Every kernel takes its sizes and constants as parameters and exists for two element
+// types: bf16 (serving) and fp32 (the exact mode: every product and sum in true 32-bit).
+//
+// Sequence metadata follows the engine's convention (api.h AttnParams): per sequence q_start (first row), q_len (rows
+// in this step, 0 = inactive) and ctx_len (tokens after this step); a row's position is ctx_len - q_len + its offset.
+#pragma once
+#include "api.h"
+
+namespace dsse {
+
+struct GemmRmParams {
+  const void* x;     // [M, K] rows ldx apart, batch z at + z * xbs elements
+  const void* w;     // [N, K] rows ldw apart (row-major [out, in]), batch z at + z * wbs
+  const void* bias;  // [N] of the weight's type or null, batch z at + z * bbs
+  void* out;         // [M, N] rows ldo apart, batch z at + z * obs; fp32 when out_f32 else the element type
+  int M, N, K, batch;
+  int ldx, ldw, ldo;
+  long long xbs, wbs, bbs, obs;
+  int act;           // 0 none, 1 gelu (tanh form)
+  int out_f32;
+  int f32;           // element type of x / w / bias: 0 bf16, 1 fp32
+  int vecx, vecw;    // 16-byte fragment loads allowed (base, row and batch strides aligned)
+};
+
+struct ScalarNormParams {
+  const float* y;    // [M, W] sublayer output (mode 0) -- unused in mode 1
+  const void* g;     // one number, element type
+  float* resid;      // [M, W] fp32 stream
+  void* xb;          // [M, W] element type: the stream's rounding (mode 0) / the normed stream (mode 1)
+  int M, W;
+  float eps;
+  int mode;          // 0: resid += y / rms(y) * g, xb = resid;  1: xb = resid / rms(resid) * g
+  int f32;
+};
+
+struct LatentKvWriteParams {
+  const float* ckr;      // [T, rk + dr] down-projection (latent | shared rotated key part)
+  const void* norm_w;    // [rk]
+  const int* positions;  // [T]
+  const int* slots;      // [T] cache row (page * kBS + offset), -1 = skip
+  const float2* rope;    // [rope_len, dr / 2] (cos, sin), amplitude folded in
+  void* cache;           // [pages * kBS, rk + dr]
+  int T, rk, dr, rope_len, num_slots;
+  float eps;
+  int f32;
+};
+
+struct LatentAttnParams {
+  const void* q;         // [T, H, dn + dr]: the rotated part is read (and rotated) here
+  const float* q_abs;    // [T, H, rk]: the unrotated part folded through the key up-projection
+  const void* cache;     // [pages * kBS, rk + dr]
+  const int* block_tables;
+  int max_blocks, num_blocks;
+  const int* q_start;
+  const int* q_len;
+  const int* ctx_len;
+  const int* work_seq;
+  const int* work_tile;
+  const float2* rope;
+  void* out;             // [T, H, rk]: softmax-weighted sum of latents (the value up-projection follows)
+  int H, dn, dr, rk, window, qt, rope_len;
+  float scale;
+  int f32;
+};
+
+struct ConvStateParams {
+  const float* in;       // [T, C] fp32
+  const void* taps;      // [C, K] (last column = the current token)
+  const void* bias;      // [C]
+  float* tail;           // [slots, K - 1, C] last K - 1 inputs of each sequence
+  const int* q_start;
+  const int* q_len;
+  const int* ctx_len;
+  const int* state_slot;
+  float* out;            // [T, C] fp32
+  void* out_b;           // [T, C] element type (the gates' GEMM input)
+  int nseq, C, K;
+  int f32;
+};
+
+struct LruScanParams {
+  const float* u;        // [T, C] convolution output
+  const float* gates;    // [T, blocks, 2 * bw]: per block [recurrence gate | input gate] pre-activations (bias added)
+  const void* y;         // [T, C] gelu branch
+  const void* lam;       // [C]
+  float* state;          // [slots, C]
+  const int* q_start;
+  const int* q_len;
+  const int* ctx_len;
+  const int* state_slot;
+  void* out;             // [T, C] element type: state * y
+  int nseq, C, bw;
+  float c;               // 8: log a = -c r softplus(lam)
+  int f32;
+};
+
+struct MoeRouterParams {
+  const void* x;         // [M, W]
+  const void* w;         // [E, W]
+  const void* b;         // [E]
+  int* topk_idx;         // [M, top]
+  float* topk_w;         // [M, top]
+  int M, W, E, top;
+  int f32;
+};
+
+struct MoeFfnParams {
+  const void* x;         // [M, W]
+  const int* topk_idx;
+  const float* topk_w;
+  const void* gate;      // [E, F, W]
+  const void* up;        // [E, F, W]
+  const void* down;      // [E, W, F]
+  const void* sgate;     // shared expert [Fs, W] or null
+  const void* sup;
+  const void* sdown;     // [W, Fs]
+  float* out;            // [M, W] fp32
+  int M, W, F, Fs, E, top;
+  int f32;
+};
+
+}  // namespace dsse
+
+extern "C" {
+hipError_t dsse_gemm_rm(const dsse::GemmRmParams* p, hipStream_t st);
+hipError_t dsse_scalar_norm(const dsse::ScalarNormParams* p, hipStream_t st);
+hipError_t dsse_embed_rows(int M, int W, int vocab, const int* ids, const void* embed, float* resid, void* xb, int f32,
+                           hipStream_t st);
+hipError_t dsse_latent_kv_write(const dsse::LatentKvWriteParams* p, hipStream_t st);
+hipError_t dsse_latent_attention(int num_work, const dsse::LatentAttnParams* p, hipStream_t st);
+hipError_t dsse_conv_state(const dsse::ConvStateParams* p, hipStream_t st);
+hipError_t dsse_lru_scan(const dsse::LruScanParams* p, hipStream_t st);
+hipError_t dsse_moe_router(const dsse::MoeRouterParams* p, hipStream_t st);
+hipError_t dsse_moe_ffn(const dsse::MoeFfnParams* p, hipStream_t st);
+}

@@ -7,6 +7,7 @@
   loadgen   Python twin of the reference demo/load-generator (producer via RESP, consumer via SSE);
             the native one is ``_lib/dsse-loadgen`` (same flags, epoll, 10k+ connections)
   build     compile the HIP kernels + native runtime in-tree
+  trace     replay a token trace through the engine and write logits (engine/trace.py; also ``bin/trace_run``)
 """
 from __future__ import annotations
 
@@ -42,6 +43,10 @@ def main(argv=None):
         from .tools_loadgen import main as lg_main
 
         return lg_main(rest)
+    if cmd == "trace":
+        from .engine.trace import main as trace_main
+
+        return trace_main(rest)
     if cmd == "build":
         from . import _build
 

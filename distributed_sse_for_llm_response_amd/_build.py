@@ -89,21 +89,23 @@ def build_kernels(verbose: bool = False, force: bool = False, variant: str | Non
     headers = sorted(kdir.glob("*.h"))
     common = ["-O3", "-std=c++17", "-fPIC", f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-Wno-unused-result"]
     common += KERNEL_VARIANTS.get(variant, [])
+    # device code without packed fp32 instructions: scalar float math only
+    nopk = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
     out_so = kernels_so(variant)
     jobs, objs = [], []
     for src in sorted(kdir.glob("*.hip")):
         obj = obj_dir / (src.stem + ".o")
         objs.append(obj)
         if force or _stale(obj, [src, *headers]):
-            jobs.append([HIPCC, f"--offload-arch={ARCH}", *common, "-munsafe-fp-atomics", "-c", src, "-o", obj])
-    bsrc = kdir / "bindings.cpp"
-    bobj = obj_dir / "bindings.o"
-    objs.append(bobj)
-    if force or _stale(bobj, [bsrc, *headers]):
-        jobs.append([
-            HIPCC, *common, "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-x", "hip", "--offload-host-only",
-            "-I", inc, "-I", api_inc, "-c", bsrc, "-o", bobj,
-        ])
+            jobs.append([HIPCC, f"--offload-arch={ARCH}", *common, *nopk, "-munsafe-fp-atomics", "-c", src, "-o", obj])
+    for bsrc in sorted(kdir.glob("bindings*.cpp")):  # torch op registrations: host-only translation units
+        bobj = obj_dir / (bsrc.stem + ".o")
+        objs.append(bobj)
+        if force or _stale(bobj, [bsrc, *headers]):
+            jobs.append([
+                HIPCC, *common, "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-x", "hip", "--offload-host-only",
+                "-I", inc, "-I", api_inc, "-c", bsrc, "-o", bobj,
+            ])
     _parallel(jobs, verbose)
     if force or _stale(out_so, objs):
         tmp = out_so.with_name(out_so.name + ".tmp")

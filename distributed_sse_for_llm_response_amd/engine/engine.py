@@ -827,6 +827,98 @@ class LLMEngine:
             elif s.produced >= s.params.max_tokens or s.orig_len + s.produced >= self.r.max_model_len:
                 self._finish(s, events, reason="length")
 
+    # ------------------------------------------------------------------ given tokens (scoring, trace replay)
+    def force_step(self, entries: list, end=()) -> "torch.Tensor | None":
+        """One engine step over GIVEN tokens instead of sampled ones: ``entries`` = [(conversation id, tokens, want)],
+        all run together as one batch; returns the fp32 logits [wanted, vocab] at the asked offsets (in the order of
+        the entries and of each ``want``), or None.  ``end``: conversations whose slot and pages are released after
+        the step.
+
+        It is the serving step with the token source swapped: a conversation is admitted at its first entry into the
+        lowest free decode slot, pages come from the engine's allocator as the sequence grows, a single next token of
+        a running sequence rides in the decode rows of the batch bucket (the captured decode graph when the step has
+        nothing else) and longer portions are prompt chunks of the same step (ModelRunner.mixed).  Tokens the step
+        samples are discarded: the next entry overwrites them.  Not to be interleaved with ``step()`` on the same
+        engine while either has sequences running."""
+        r = self.r
+        dec, chunks, order = [], [], []
+        for cid, tokens, want in entries:
+            s = self.by_conv.get(cid)
+            if s is None:
+                free = next((i for i, x in enumerate(self.slots) if x is None), -1)
+                if free < 0:
+                    raise RuntimeError(f"no free decode slot for {cid!r} ({r.max_batch} sequences are live)")
+                s = Sequence(rid=next(self._rid), conversation_id=cid, prompt=[], slot=free, state="prefill",
+                             params=SamplingParams(temperature=0.0, max_tokens=2 ** 30, ignore_eos=True))
+                self.slots[free] = s
+                self.by_conv[cid] = s
+            n, pos0 = len(tokens), s.prefilled
+            if n == 0:
+                continue
+            if pos0 + n > r.max_model_len:
+                raise RuntimeError(f"{cid!r}: {pos0 + n} tokens exceed the engine's context of {r.max_model_len}")
+            need = blocks_needed(pos0 + n) - len(s.blocks)
+            if need > 0:
+                s.blocks = s.blocks + self.alloc.allocate(need)
+            self._dirty_slots.add(s.slot)
+            s.prompt = s.prompt + list(tokens)
+            if n == 1 and pos0 > 0:
+                if list(want) not in ([], [0]):
+                    raise ValueError(f"{cid!r}: a single token has offset 0 only")
+                s.state = "decode"
+                dec.append((s, int(tokens[0]), pos0))
+                order.append(("d", s.slot, bool(want)))
+            else:
+                s.state = "prefill"
+                chunks.append(PrefillSeq(slot=s.slot, tokens=list(tokens), start_pos=pos0, block_table=s.blocks,
+                                         last_chunk=False, want=tuple(int(o) for o in want)))
+                order.append(("c", len(chunks) - 1, len(want)))
+            s.prefilled = pos0 + n
+        # sequences left out of this step hold: not in the decode rows (their slots stay inactive)
+        live = {s.slot for s, _, _ in dec}
+        for x in self.slots:
+            if x is not None and x.slot not in live and x.state == "decode":
+                x.state = "prefill"
+                self._dirty_slots.add(x.slot)
+        self._upload()
+        B = 0
+        if dec:
+            B = next(b for b in batch_buckets(r.max_batch) if b >= max(s.slot for s, _, _ in dec) + 1)
+            idx = torch.tensor([[s.slot for s, _, _ in dec], [t for _, t, _ in dec], [p for _, _, p in dec]],
+                               dtype=torch.long)
+            if r.device.type == "cuda":
+                idx = idx.pin_memory().to(r.device, non_blocking=True)
+            r.ids.index_copy_(0, idx[0], idx[1].to(torch.int32))
+            r.positions.index_copy_(0, idx[0], idx[2].to(torch.int32))
+        row = self.ring_head % RING_SIZE
+        if dec and chunks:
+            r.mixed(B, chunks, ring_row=row)
+            self.stats["mixed_steps"] += 1
+        elif dec:
+            r.decode(B)
+            self.stats["decode_steps"] += 1
+        elif chunks:
+            r.prefill(chunks, ring_row=row)
+            from .. import ops
+            ops.ring_advance(r.ring_counter)
+        if dec or chunks:
+            self.ring_head += 1
+            self.step_no += 1
+            self.stats["steps"] += 1
+        out, k = [], 0
+        for kind, i, w in order:
+            if kind == "d":
+                if w:
+                    out.append(r.logits[i:i + 1])
+            elif w:
+                out.append(r.kept_logits[k:k + w])
+                k += w
+        for cid in end:
+            s = self.by_conv.get(cid)
+            if s is not None:
+                self._finish(s, [], reason="stop")
+        return torch.cat(out) if out else None
+
     def fail_all(self, text: str = "[ERROR]") -> list:
         """Terminal `text` events for every live conversation (running, paused, queued), after an EngineFault: the
         clients see the reference's upstream-error token (llm-stream-proxy main.go:166-186) instead of a hang or

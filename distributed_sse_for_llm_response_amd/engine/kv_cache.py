@@ -57,3 +57,41 @@ class BlockAllocator:
 
 def blocks_needed(num_tokens: int) -> int:
     return (num_tokens + PAGE - 1) // PAGE
+
+
+class LatentKVCache:
+    """Paged cache of latent-attention layers: one row [normed latent (rank) | rotated shared key part (rot)] per
+    token, nothing per head.  One tensor per attention layer, [blocks, PAGE, rank + rot] in the engine's element
+    type; layers index it with the same block tables (a page id means the same page in every layer), so the host
+    allocator and the block tables are the ones the dense KV cache uses.  ``widths`` maps layer index -> rank + rot
+    (layers without attention have no entry)."""
+
+    def __init__(self, widths: dict, num_blocks: int, device, dtype=torch.bfloat16):
+        self.num_blocks = num_blocks
+        self.layers = {li: torch.zeros(num_blocks, PAGE, w, device=device, dtype=dtype) for li, w in widths.items()}
+
+    def __getitem__(self, li: int) -> torch.Tensor:
+        return self.layers[li]
+
+    @staticmethod
+    def bytes_per_block(widths: dict, elem_bytes: int = 2) -> int:
+        return max(1, sum(widths.values()) * PAGE * elem_bytes)
+
+
+class RecurrentStateCache:
+    """Per-sequence state of recurrent layers, indexed by the engine's decode slot (a sequence owns one slot from
+    admission to its end, so the slot is also its state slot): per layer the fp32 recurrence state [slots, C] and the
+    convolution tail [slots, taps - 1, C] (the last taps - 1 inputs).  Nothing is cleared when a slot changes hands:
+    the kernels start a sequence whose first row is position 0 from zeros.  ``shapes`` maps layer index -> (C, taps)."""
+
+    def __init__(self, shapes: dict, num_slots: int, device):
+        self.num_slots = num_slots
+        self.state = {li: torch.zeros(num_slots, c, device=device, dtype=torch.float32) for li, (c, _) in shapes.items()}
+        self.tail = {li: torch.zeros(num_slots, k - 1, c, device=device, dtype=torch.float32)
+                     for li, (c, k) in shapes.items()}
+
+    def move(self, src_idx: torch.Tensor, dst_idx: torch.Tensor) -> None:
+        """State of slot src[i] -> slot dst[i] (gathered before it is scattered, so swaps work)."""
+        for group in (self.state, self.tail):
+            for t in group.values():
+                t.index_copy_(0, dst_idx, t.index_select(0, src_idx))

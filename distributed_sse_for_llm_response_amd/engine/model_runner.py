@@ -185,9 +185,157 @@ class PrefillSeq:
     start_pos: int          # absolute position of tokens[0]
     block_table: list       # the sequence's full block table
     last_chunk: bool        # sample a token after this chunk
+    want: tuple = ()        # offsets in this chunk whose logits the caller keeps (RunnerBase.kept_logits)
 
 
-class ModelRunner:
+class RunnerBase:
+    """What every model runner shares with the engine (engine.py): the slot-indexed decode state on the device (last
+    token, position, sampling parameters, block tables), the token ring, the logits -> candidates -> pick sampling with
+    its commit, first-token sampling after a prompt's last chunk, slot compaction and the captured-graph replay.  A
+    runner adds its model's forward passes: ``decode_forward(B)``, ``prefill(seqs, ring_row)`` and (optionally)
+    ``mixed(B, seqs, ring_row)``, a ``kv`` object with ``num_blocks``, and ``_lm_head(rows, logits)``."""
+
+    def _init_slots(self, Bm: int, max_blocks: int, V: int, dev, comm) -> None:
+        i32 = dict(device=dev, dtype=torch.int32)
+        # ---- decode state (slot-indexed, device resident) ----
+        self.ids = torch.zeros(Bm, **i32)
+        self.positions = torch.zeros(Bm, **i32)
+        # per-slot sampling state in ONE int32 buffer [active | temperature | top_k | top_p | seeds (Bm x 2)] (the
+        # float fields are views of their words): the engine uploads a changed slot set with one pinned copy
+        # (LLMEngine._upload)
+        self.slot_meta = torch.zeros(6 * Bm, **i32)
+        self.active = self.slot_meta[:Bm]
+        self.block_tables = torch.zeros(Bm, max_blocks, **i32)
+        self.slots = torch.full((Bm,), -1, **i32)
+        self.ctx_len = torch.zeros(Bm, **i32)
+        self.q_len = torch.zeros(Bm, **i32)
+        self.q_start = torch.arange(Bm, **i32)
+        self.work_seq = torch.arange(Bm, **i32)
+        self.work_tile = torch.zeros(Bm, **i32)
+        self.temperature = self.slot_meta[Bm:2 * Bm].view(torch.float32)
+        self.top_k = self.slot_meta[2 * Bm:3 * Bm]
+        self.top_p = self.slot_meta[3 * Bm:4 * Bm].view(torch.float32)
+        self.top_p.fill_(1.0)
+        self.seeds = self.slot_meta[4 * Bm:].view(Bm, 2)
+        self.ring = torch.zeros(RING_SIZE, Bm, **i32)
+        self.ring_counter = torch.zeros(1, **i32)
+        self.health = torch.zeros(4, device=dev, dtype=torch.int32)
+        self.logits = torch.zeros(Bm, V, device=dev, dtype=torch.float32)
+        nch = SAMPLE_CHUNKS if dev.type == "cuda" else 1
+        self._cand = {b: torch.zeros(b, nch, 2, device=dev, dtype=torch.float32) for b in batch_buckets(Bm)}
+        self._cand_all = {b: torch.zeros(comm.size, b, nch, 2, device=dev, dtype=torch.float32)
+                          for b in batch_buckets(Bm)}
+        self.graphs = {}
+        self.graph_pool = None
+        self.kept_logits = None
+
+    def _sample_commit(self, B: int) -> None:
+        """Candidates per (row, vocab chunk) on each rank -> (TP: all-gather, 8 B per candidate) -> pick."""
+        r = slice(0, B)
+        cand = self._cand[B]
+        ops.sample_candidates(self.logits[r], self.temperature[r], self.top_k[r], self.top_p[r], self.seeds[r],
+                              self.positions[r], self.active[r], cand, self.w.vocab_offset)
+        if self.comm.size == 1:
+            cand_all = cand.unsqueeze(0)
+        else:
+            cand_all = self._cand_all[B]
+            self.comm.all_gather_into(cand_all, cand)
+        ops.sample_pick(cand_all, self.active[r], self.ids[r], self.ring, self.ring_counter, self.positions[r],
+                        vocab=self.cfg.vocab_size)
+
+    def health_faults(self, words) -> list:
+        """Descriptions of the nonzero health words in `words` (a host copy of self.health)."""
+        return [HEALTH_WORDS[i] for i in range(min(len(HEALTH_WORDS), len(words))) if int(words[i]) != 0]
+
+    def bucket_for(self, n_active_max_slot: int) -> int:
+        for b in batch_buckets(self.max_batch):
+            if b >= n_active_max_slot:
+                return b
+        return self.max_batch
+
+    def _snapshot_state(self):
+        return [t.clone() for t in (self.ids, self.positions, self.ring, self.ring_counter)]
+
+    def _restore_state(self, saved):
+        for t, s in zip((self.ids, self.positions, self.ring, self.ring_counter), saved):
+            t.copy_(s)
+
+    def move_slots(self, src: list, dst: list) -> None:
+        """Slot compaction: decode state (last token, position) of slot src[i] -> dst[i], gathered before it
+        is scattered so swaps work; stream-ordered after every decode step already enqueued."""
+        idx = torch.tensor([src, dst], dtype=torch.long)
+        if self.device.type == "cuda":  # pinned + non_blocking: no host wait for the decode steps already queued
+            idx = idx.pin_memory().to(self.device, non_blocking=True)
+        si, di = idx[0], idx[1]
+        for t in (self.ids, self.positions):
+            t.index_copy_(0, di, t.index_select(0, si))
+
+    def decode(self, B: int) -> None:
+        g = self.graphs.get(B)
+        if g is not None:
+            g.replay()
+        else:
+            self.decode_forward(B)
+
+    def _prefill_sample(self, seqs: list, x, q_start: list, q_len: list, ring_row: int) -> None:
+        """Sequences whose last chunk this is sample their first token (rows q_start + q_len - 1 of `x`) into
+        ids[slot] and ring[ring_row, slot]; positions[slot] is set on the device."""
+        w, cfg, comm, dev = self.w, self.cfg, self.comm, self.device
+        last = [i for i, s in enumerate(seqs) if s.last_chunk]
+        if not last:
+            return
+        f32 = dict(device=dev, dtype=torch.float32)
+        nL = len(last)
+        # one pinned, non-blocking upload of the three index vectors: a pageable torch.tensor(..., device=dev) is a
+        # synchronous copy that waits for every step already queued (the prefill graph and the pipelined decode
+        # steps) -- 27-30 ms of host stall per prompt at ~120 streams (profiles/r3/serving_trace.md)
+        idx = torch.tensor([q_start[i] + q_len[i] - 1 for i in last] + [seqs[i].slot for i in last] +
+                           [seqs[i].start_pos + len(seqs[i].tokens) - 1 for i in last], dtype=torch.long)
+        if dev.type == "cuda":
+            idx = idx.pin_memory().to(dev, non_blocking=True)
+        rows, slot_idx, last_pos = idx[:nL], idx[nL:2 * nL], idx[2 * nL:].to(torch.int32)
+        xl = x.index_select(0, rows)
+        logits = torch.empty(nL, w.vocab_local, **f32)
+        self._lm_head(xl, logits)
+        new_ids = torch.zeros(nL, dtype=torch.int32, device=dev)
+        temp = self.temperature.index_select(0, slot_idx)
+        tk = self.top_k.index_select(0, slot_idx)
+        tp = self.top_p.index_select(0, slot_idx)
+        sd = self.seeds.index_select(0, slot_idx).contiguous()
+        nch = SAMPLE_CHUNKS if dev.type == "cuda" else 1
+        cand = torch.zeros(nL, nch, 2, **f32)
+        ops.sample_candidates(logits, temp, tk, tp, sd, last_pos, None, cand, w.vocab_offset)
+        if comm.size == 1:
+            cand_all = cand.unsqueeze(0)
+        else:
+            cand_all = torch.zeros(comm.size, nL, nch, 2, **f32)
+            comm.all_gather_into(cand_all, cand)
+        ops.sample_pick(cand_all, None, new_ids, vocab=cfg.vocab_size)
+        self.ids.index_copy_(0, slot_idx, new_ids)
+        self.ring[ring_row].index_copy_(0, slot_idx, new_ids)
+        self.positions.index_copy_(0, slot_idx, last_pos + 1)
+
+    def _keep_logits(self, seqs: list, x, q_start: list) -> None:
+        """kept_logits [n, V] (fp32) = the logits of the rows that chunks ask for (PrefillSeq.want), in the order of
+        `seqs` and of each chunk's `want`; None when no chunk asks.  Scoring a given continuation (teacher forcing)
+        reads them; sampling does not."""
+        rows = [q_start[i] + o for i, s in enumerate(seqs) for o in s.want]
+        self.kept_logits = None
+        if not rows:
+            return
+        idx = torch.tensor(rows, dtype=torch.long)
+        if self.device.type == "cuda":
+            idx = idx.pin_memory().to(self.device, non_blocking=True)
+        self.kept_logits = torch.empty(len(rows), self.w.vocab_local, device=self.device, dtype=torch.float32)
+        self._lm_head(x.index_select(0, idx), self.kept_logits)
+
+    def _lm_head(self, rows, logits) -> None:
+        """logits (fp32) of the given rows of the stream a prompt pass leaves (the runner's final norm included when
+        the stream is not normed yet)."""
+        raise NotImplementedError
+
+
+class ModelRunner(RunnerBase):
     def __init__(self, w: EngineWeights, num_blocks: int, max_batch: int = 64, max_model_len: int = 4096,
                  max_prefill_tokens: int = 8192, device="cuda", comm: TPComm | None = None, use_graphs=None):
         self.w, self.cfg = w, w.cfg
@@ -204,29 +352,7 @@ class ModelRunner:
         self.kv = KVCache(cfg.num_layers, num_blocks, nkv, dev)
         self.rope = rope_table(max(cfg.max_position, max_model_len + 1), cfg.rope_theta, dev)
         Bm = max_batch
-        i32 = dict(device=dev, dtype=torch.int32)
-        # ---- decode state (slot-indexed, device resident) ----
-        self.ids = torch.zeros(Bm, **i32)
-        self.positions = torch.zeros(Bm, **i32)
-        # per-slot sampling state in ONE int32 buffer [active | temperature | top_k | top_p | seeds (Bm x 2)] (the
-        # float fields are views of their words): the engine uploads a changed slot set with one pinned copy
-        # (LLMEngine._upload)
-        self.slot_meta = torch.zeros(6 * Bm, **i32)
-        self.active = self.slot_meta[:Bm]
-        self.block_tables = torch.zeros(Bm, self.max_blocks, **i32)
-        self.slots = torch.full((Bm,), -1, **i32)
-        self.ctx_len = torch.zeros(Bm, **i32)
-        self.q_len = torch.zeros(Bm, **i32)
-        self.q_start = torch.arange(Bm, **i32)
-        self.work_seq = torch.arange(Bm, **i32)
-        self.work_tile = torch.zeros(Bm, **i32)
-        self.temperature = self.slot_meta[Bm:2 * Bm].view(torch.float32)
-        self.top_k = self.slot_meta[2 * Bm:3 * Bm]
-        self.top_p = self.slot_meta[3 * Bm:4 * Bm].view(torch.float32)
-        self.top_p.fill_(1.0)
-        self.seeds = self.slot_meta[4 * Bm:].view(Bm, 2)
-        self.ring = torch.zeros(RING_SIZE, Bm, **i32)
-        self.ring_counter = torch.zeros(1, **i32)
+        self._init_slots(Bm, self.max_blocks, V, dev, self.comm)
         # ---- decode activations ----
         bf = dict(device=dev, dtype=torch.bfloat16)
         self.resid = torch.zeros(Bm, H, device=dev, dtype=torch.float32)
@@ -241,12 +367,6 @@ class ModelRunner:
         if torch.device(dev).type == "cuda":
             slab_floats = max(slab_floats, 8 * min(PREFILL_SLAB_ROWS, max_prefill_tokens) * H)
         self.split_part = torch.zeros(slab_floats, device=dev, dtype=torch.float32)
-        self.health = torch.zeros(4, device=dev, dtype=torch.int32)
-        self.logits = torch.zeros(Bm, V, device=dev, dtype=torch.float32)
-        nch = SAMPLE_CHUNKS if dev.type == "cuda" else 1
-        self._cand = {b: torch.zeros(b, nch, 2, device=dev, dtype=torch.float32) for b in batch_buckets(Bm)}
-        self._cand_all = {b: torch.zeros(self.comm.size, b, nch, 2, device=dev, dtype=torch.float32)
-                          for b in batch_buckets(Bm)}
         part, nparts = decode_partitioning(1, nkv, max_model_len)
         ws = max(decode_partitioning(b, nkv, max_model_len)[1] * b for b in batch_buckets(Bm))
         self.part_o = torch.zeros(max(1, ws) * nkv * 16 * 128, device=dev, dtype=torch.float32)
@@ -259,12 +379,13 @@ class ModelRunner:
         if self.comm.size > 1 and self.comm.rank == 0:
             print(f"[engine] TP={self.comm.size} decode all-reduce + candidate all-gather: "
                   f"{'IPC kernels' if not self.fast_ar_reason else 'RCCL (' + self.fast_ar_reason + ')'}", flush=True)
-        self.graphs = {}
-        self.graph_pool = None
         self.pf_graphs = {}   # row bucket -> captured prefill graph
         self.pf = None        # static prefill buffers (allocated by capture)
         self.mx_graphs = {}   # decode bucket B -> [(chunk rows C, captured mixed prefill + decode graph)], C ascending
         self.host_trace = None  # a list: host seconds of each graph-replayed mixed step (upload, replay, sampling)
+
+    def _lm_head(self, rows, logits) -> None:
+        ops.gemm_out(rows, self.w.lm_head_t, logits)
 
     # ------------------------------------------------------------------ decode
     def decode_forward(self, B: int) -> None:
@@ -345,24 +466,6 @@ class ModelRunner:
             ops.gemm_out(a, wt, tmp)
             self.comm.all_reduce_rmsnorm(tmp, resid, norm_w, x, eps)
 
-    def _sample_commit(self, B: int) -> None:
-        """Candidates per (row, vocab chunk) on each rank -> (TP: all-gather, 8 B per candidate) -> pick."""
-        r = slice(0, B)
-        cand = self._cand[B]
-        ops.sample_candidates(self.logits[r], self.temperature[r], self.top_k[r], self.top_p[r], self.seeds[r],
-                              self.positions[r], self.active[r], cand, self.w.vocab_offset)
-        if self.comm.size == 1:
-            cand_all = cand.unsqueeze(0)
-        else:
-            cand_all = self._cand_all[B]
-            self.comm.all_gather_into(cand_all, cand)
-        ops.sample_pick(cand_all, self.active[r], self.ids[r], self.ring, self.ring_counter, self.positions[r],
-                        vocab=self.cfg.vocab_size)
-
-    def health_faults(self, words) -> list:
-        """Descriptions of the nonzero health words in `words` (a host copy of self.health)."""
-        return [HEALTH_WORDS[i] for i in range(min(len(HEALTH_WORDS), len(words))) if int(words[i]) != 0]
-
     def close(self) -> None:
         """Release the TP all-reduce's IPC mappings and buffer.  Collective over the TP group: the device is
         synchronised, then every rank passes a barrier, so no peer's kernel can still be reading this rank's buffer
@@ -376,12 +479,6 @@ class ModelRunner:
                 print(f"[engine] TP rank {self.comm.rank}: barrier before the IPC teardown failed ({e})", flush=True)
             self.comm.fast_ar.close()
             self.comm.fast_ar = None
-
-    def bucket_for(self, n_active_max_slot: int) -> int:
-        for b in batch_buckets(self.max_batch):
-            if b >= n_active_max_slot:
-                return b
-        return self.max_batch
 
     def _collectives_capturable(self) -> tuple:
         """TP>1 startup self-check: an all-reduce captured into a graph and replayed must produce the sum on
@@ -549,30 +646,6 @@ class ModelRunner:
         or None (the step runs eagerly)."""
         return next((c for c, _ in self.mx_graphs.get(B, ()) if c >= T), None)
 
-    def _snapshot_state(self):
-        return [t.clone() for t in (self.ids, self.positions, self.ring, self.ring_counter)]
-
-    def _restore_state(self, saved):
-        for t, s in zip((self.ids, self.positions, self.ring, self.ring_counter), saved):
-            t.copy_(s)
-
-    def move_slots(self, src: list, dst: list) -> None:
-        """Slot compaction: decode state (last token, position) of slot src[i] -> dst[i], gathered before it
-        is scattered so swaps work; stream-ordered after every decode step already enqueued."""
-        idx = torch.tensor([src, dst], dtype=torch.long)
-        if self.device.type == "cuda":  # pinned + non_blocking: no host wait for the decode steps already queued
-            idx = idx.pin_memory().to(self.device, non_blocking=True)
-        si, di = idx[0], idx[1]
-        for t in (self.ids, self.positions):
-            t.index_copy_(0, di, t.index_select(0, si))
-
-    def decode(self, B: int) -> None:
-        g = self.graphs.get(B)
-        if g is not None:
-            g.replay()
-        else:
-            self.decode_forward(B)
-
     # ------------------------------------------------------------------ prefill
     def _proj(self, a, wt, out) -> None:
         """out = a·wᵀ in bf16 on the engine's tiled-layout GEMMs (every row count: no library GEMM)."""
@@ -739,44 +812,6 @@ class ModelRunner:
         d["fslots"] = plan[2] if plan else 0
         return T, q_start, q_len, ctx_len, d
 
-    def _prefill_sample(self, seqs: list, x, q_start: list, q_len: list, ring_row: int) -> None:
-        """Sequences whose last chunk this is sample their first token (rows q_start + q_len - 1 of `x`) into
-        ids[slot] and ring[ring_row, slot]; positions[slot] is set on the device."""
-        w, cfg, comm, dev = self.w, self.cfg, self.comm, self.device
-        last = [i for i, s in enumerate(seqs) if s.last_chunk]
-        if not last:
-            return
-        f32 = dict(device=dev, dtype=torch.float32)
-        nL = len(last)
-        # one pinned, non-blocking upload of the three index vectors: a pageable torch.tensor(..., device=dev) is a
-        # synchronous copy that waits for every step already queued (the prefill graph and the pipelined decode
-        # steps) -- 27-30 ms of host stall per prompt at ~120 streams (profiles/r3/serving_trace.md)
-        idx = torch.tensor([q_start[i] + q_len[i] - 1 for i in last] + [seqs[i].slot for i in last] +
-                           [seqs[i].start_pos + len(seqs[i].tokens) - 1 for i in last], dtype=torch.long)
-        if dev.type == "cuda":
-            idx = idx.pin_memory().to(dev, non_blocking=True)
-        rows, slot_idx, last_pos = idx[:nL], idx[nL:2 * nL], idx[2 * nL:].to(torch.int32)
-        xl = x.index_select(0, rows)
-        logits = torch.empty(nL, w.vocab_local, **f32)
-        ops.gemm_out(xl, w.lm_head_t, logits)
-        new_ids = torch.zeros(nL, dtype=torch.int32, device=dev)
-        temp = self.temperature.index_select(0, slot_idx)
-        tk = self.top_k.index_select(0, slot_idx)
-        tp = self.top_p.index_select(0, slot_idx)
-        sd = self.seeds.index_select(0, slot_idx).contiguous()
-        nch = SAMPLE_CHUNKS if dev.type == "cuda" else 1
-        cand = torch.zeros(nL, nch, 2, **f32)
-        ops.sample_candidates(logits, temp, tk, tp, sd, last_pos, None, cand, w.vocab_offset)
-        if comm.size == 1:
-            cand_all = cand.unsqueeze(0)
-        else:
-            cand_all = torch.zeros(comm.size, nL, nch, 2, **f32)
-            comm.all_gather_into(cand_all, cand)
-        ops.sample_pick(cand_all, None, new_ids, vocab=cfg.vocab_size)
-        self.ids.index_copy_(0, slot_idx, new_ids)
-        self.ring[ring_row].index_copy_(0, slot_idx, new_ids)
-        self.positions.index_copy_(0, slot_idx, last_pos + 1)
-
     def prefill(self, seqs: list, ring_row: int) -> None:
         """Run one packed prefill batch: a captured graph of the smallest row bucket that holds it (metadata
         uploaded into the static buffers first), else eagerly.  Sequences whose last chunk this is sample their
@@ -802,6 +837,7 @@ class ModelRunner:
                  qkv=torch.empty(T, (nh + 2 * nkv) * 128, **bf), part=math.ceil(max(ctx_len) / 32) * 32)
         self._prefill_layers(T, d)
         self._prefill_sample(seqs, d["x"], q_start, q_len, ring_row)
+        self._keep_logits(seqs, d["x"], q_start)
 
     def _prefill_layers(self, T: int, d: dict) -> None:
         """Embedding + every layer over T packed prompt rows (buffers and metadata in `d`; graph-capturable)."""
@@ -888,6 +924,7 @@ class ModelRunner:
                  mx_slots=torch.empty(M, dtype=torch.int32, device=dev))
         self._mixed_body(B, T, d)
         self._prefill_sample(seqs, d["x"], q_start, q_len, ring_row)
+        self._keep_logits(seqs, d["x"], q_start)
 
     def _mixed_layers(self, B: int, C: int) -> None:
         """The graph body of a mixed step: bucket B decode rows + C static prompt rows (_PrefillStatic)."""

@@ -193,3 +193,142 @@ def load_safetensors(cfg: MistralConfig, path: str, tp_rank: int = 0, tp_size: i
             "down": tensors[p + "mlp.down_proj.weight"],
         })
     return convert_standard(cfg, std, tp_rank, tp_size, device)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Configuration-driven designs (models/muderax.py): row-major weights for the general GEMM (ops.gemm_rm), regrouped so
+# that every per-head / per-block / per-expert family is ONE tensor with a batch axis.
+@dataclass
+class LatentAttentionWeights:
+    q: torch.Tensor          # [H (dn + dr), W]
+    dkv: torch.Tensor        # [rk + dr, W]
+    dkv_norm: torch.Tensor   # [rk]
+    uk_t: torch.Tensor       # [H, rk, dn]: the key up-projection transposed per head (folds into the query)
+    uv: torch.Tensor         # [H, dv, rk]
+    o: torch.Tensor          # [W, H dv]
+
+
+@dataclass
+class RglruWeights:
+    y: torch.Tensor          # [C, W]
+    y_b: torch.Tensor
+    x: torch.Tensor          # [C, W]
+    x_b: torch.Tensor
+    conv: torch.Tensor       # [C, taps]
+    conv_b: torch.Tensor
+    gates: torch.Tensor      # [blocks, 2 bw, bw]: rows [recurrence gate | input gate] of each block
+    gates_b: torch.Tensor    # [blocks, 2 bw]
+    lam: torch.Tensor        # [C]
+    o: torch.Tensor          # [W, C]
+
+
+@dataclass
+class MoeWeights:
+    router: torch.Tensor     # [E, W]
+    router_b: torch.Tensor   # [E]
+    gate: torch.Tensor       # [E, F, W]
+    up: torch.Tensor         # [E, F, W]
+    down: torch.Tensor       # [E, W, F]
+    sgate: torch.Tensor = None   # shared expert [Fs, W] (None: the design has none)
+    sup: torch.Tensor = None
+    sdown: torch.Tensor = None   # [W, Fs]
+
+
+@dataclass
+class LayeredLayer:
+    norm1: torch.Tensor      # one number
+    mix: object
+    norm2: torch.Tensor = None
+    mlp: MoeWeights = None
+
+
+@dataclass
+class LayeredWeights:
+    cfg: object
+    embed: torch.Tensor
+    layers: list             # one entry per layer; layers that borrow weights hold the lender's object
+    final_norm: torch.Tensor
+    head: torch.Tensor
+    dtype: torch.dtype = torch.bfloat16
+    tp_rank: int = 0
+    tp_size: int = 1
+
+    @property
+    def vocab_local(self) -> int:
+        return self.cfg.vocab_size
+
+    @property
+    def vocab_offset(self) -> int:
+        return 0
+
+    def nbytes(self) -> int:
+        seen, n = set(), 0
+        for L in self.layers:
+            if id(L) in seen:
+                continue
+            seen.add(id(L))
+            for obj in (L, L.mix, L.mlp):
+                if obj is not None:
+                    n += sum(t.numel() * t.element_size() for t in vars(obj).values() if isinstance(t, torch.Tensor))
+        return n + sum(t.numel() * t.element_size() for t in (self.embed, self.final_norm, self.head))
+
+
+@torch.no_grad()
+def convert_layered(cfg, tensors: dict, device="cpu", dtype=torch.bfloat16) -> LayeredWeights:
+    """Checkpoint tensors {name: tensor} (models/muderax.py tensor_shapes) -> the engine's grouped layout in `dtype`
+    (bf16 for serving; fp32 is the exact mode -- bf16 checkpoint values convert without loss)."""
+    from ..models.muderax import tensor_shapes
+
+    for name, shape in tensor_shapes(cfg).items():
+        if name not in tensors:
+            raise KeyError(f"checkpoint lacks tensor {name!r}")
+        if tuple(tensors[name].shape) != tuple(shape):
+            raise ValueError(f"tensor {name!r} has shape {tuple(tensors[name].shape)}, the configuration says {shape}")
+
+    def t(name):
+        return tensors[name].to(device=device, dtype=dtype).contiguous()
+
+    def one(name):
+        return t(name).reshape(1)
+
+    own = {}
+    for i, L in enumerate(cfg.layers):
+        if L.weights_of != i:
+            continue
+        p, m = f"l{i}.", L.mixer
+        if L.kind == "latent_attention":
+            mix = LatentAttentionWeights(
+                q=t(p + "mix.q"), dkv=t(p + "mix.dkv"), dkv_norm=t(p + "mix.dkv.norm"),
+                uk_t=t(p + "mix.uk").view(m.heads, m.dim, m.kv_rank).transpose(1, 2).contiguous(),
+                uv=t(p + "mix.uv").view(m.heads, m.vdim, m.kv_rank).contiguous(), o=t(p + "mix.o"))
+        else:
+            mix = RglruWeights(
+                y=t(p + "mix.y"), y_b=t(p + "mix.y.b"), x=t(p + "mix.x"), x_b=t(p + "mix.x.b"), conv=t(p + "mix.conv"),
+                conv_b=t(p + "mix.conv.b"), gates=torch.cat([t(p + "mix.ra"), t(p + "mix.ri")], dim=1).contiguous(),
+                gates_b=torch.cat([t(p + "mix.ra.b"), t(p + "mix.ri.b")], dim=1).contiguous(), lam=t(p + "mix.lam"),
+                o=t(p + "mix.o"))
+        layer = LayeredLayer(norm1=one(p + "norm1"), mix=mix)
+        if L.mlp is not None:
+            f = L.mlp
+            stack = lambda leaf: torch.stack([t(f"{p}mlp.e{e}.{leaf}") for e in range(f.experts)]).contiguous()  # noqa: E731
+            layer.norm2 = one(p + "norm2")
+            layer.mlp = MoeWeights(router=t(p + "mlp.router"), router_b=t(p + "mlp.router.b"), gate=stack("gate"),
+                                   up=stack("up"), down=stack("down"))
+            if f.shared_ff:
+                layer.mlp.sgate, layer.mlp.sup, layer.mlp.sdown = (t(f"{p}mlp.shared.{leaf}")
+                                                                   for leaf in ("gate", "up", "down"))
+        own[i] = layer
+    return LayeredWeights(cfg=cfg, embed=t("embed"), layers=[own[L.weights_of] for L in cfg.layers],
+                          final_norm=one("final.norm"), head=t("head"), dtype=dtype)
+
+
+def load_layered_dir(cfg, path: str, device="cpu", dtype=torch.bfloat16) -> LayeredWeights:
+    """``*.safetensors`` of a checkpoint directory -> LayeredWeights (the loader executes nothing from the files)."""
+    from pathlib import Path
+
+    from safetensors.torch import load_file
+
+    tensors = {}
+    for f in sorted(Path(path).glob("*.safetensors")):
+        tensors.update(load_file(str(f)))
+    return convert_layered(cfg, tensors, device=device, dtype=dtype)

@@ -277,3 +277,7 @@ def kernel_checks(clear: bool = True, raise_on_error: bool = True) -> list:
         raise KernelCheckError("; ".join(f"{f}:{ln} index {v} not below {b} ({n} times)" for f, ln, v, b, n in bad))
     return bad
 
+
+
+from .layers import (conv_state, embed_rows, gemm_rm, latent_attention, latent_kv_write, lru_scan,  # noqa: E402,F401
+                     moe_ffn, moe_router, scalar_norm)

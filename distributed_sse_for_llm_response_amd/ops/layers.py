@@ -1,0 +1,96 @@
+"""Layer-mechanism ops for configuration-driven designs: HIP kernels on GPU tensors, ``layers_reference`` on CPU tensors.
+
+Dispatch follows ``ops/__init__.py``: a GPU tensor always takes the HIP kernel (the call raises when the kernel library
+is missing), a CPU tensor the PyTorch reference.  The element type (bf16, or fp32 for the exact mode) comes with the
+tensors; sizes and constants are arguments, so another design reuses the same ops with its own numbers.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import layers_reference as lref
+
+
+def _hip(t: torch.Tensor) -> bool:
+    if t.is_cuda:
+        from . import load_library
+
+        load_library(required=True)
+        return True
+    return False
+
+
+def gemm_rm(x, w, out, bias=None, act: int = 0):
+    """out = act(x · wᵀ + bias) for row-major w [N, K]; any sizes; 3-D operands are batched over dim 0 (strided views
+    of wider buffers are fine: only the innermost stride must be 1).  act: 0 none, 1 gelu (tanh form)."""
+    if _hip(x):
+        torch.ops.dsse.gemm_rm(x, w, out, bias, act)
+    else:
+        lref.gemm_rm(x, w, out, bias, act)
+
+
+def scalar_norm(y, g, resid, xb, eps: float):
+    """y given: resid += y / rms(y) · g (one number g), xb = resid rounded.  y None: xb = resid / rms(resid) · g."""
+    if _hip(resid):
+        torch.ops.dsse.scalar_norm(y, g, resid, xb, eps)
+    else:
+        lref.scalar_norm(y, g, resid, xb, eps)
+
+
+def embed_rows(ids, embed, resid, xb):
+    """resid (fp32) = xb = embed[ids]."""
+    if _hip(resid):
+        torch.ops.dsse.embed_rows(ids, embed, resid, xb)
+    else:
+        lref.embed_rows(ids, embed, resid, xb)
+
+
+def latent_kv_write(ckr, norm_w, positions, slots, rope, cache, eps: float):
+    """cache[slot] = [rms-norm(ckr[:, :rk]) · norm_w | rot(ckr[:, rk:])] for rows with slot >= 0."""
+    if _hip(ckr):
+        torch.ops.dsse.latent_kv_write(ckr, norm_w, positions, slots, rope, cache, eps)
+    else:
+        lref.latent_kv_write(ckr, norm_w, positions, slots, rope, cache, eps)
+
+
+def latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile, rope, out,
+                     window: int, scale: float, qt: int):
+    """Sliding-window multi-query attention over the latent cache (folded form), `qt` query rows per work item."""
+    if _hip(q):
+        torch.ops.dsse.latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile,
+                                        rope, out, window, scale, qt)
+    else:
+        lref.latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile, rope, out,
+                              window, scale, qt)
+
+
+def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b):
+    """Per-channel causal convolution continued from each sequence's slot tail (and the tail's update)."""
+    if _hip(inp):
+        torch.ops.dsse.conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b)
+    else:
+        lref.conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b)
+
+
+def lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, c: float):
+    """Real-gated linear recurrence continued from each sequence's slot state; out = state · y."""
+    if _hip(u):
+        torch.ops.dsse.lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, c)
+    else:
+        lref.lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, c)
+
+
+def moe_router(x, w, b, topk_idx, topk_w):
+    """fp32 router logits, the top-k experts per row and the softmax over the chosen logits."""
+    if _hip(x):
+        torch.ops.dsse.moe_router(x, w, b, topk_idx, topk_w)
+    else:
+        lref.moe_router(x, w, b, topk_idx, topk_w)
+
+
+def moe_ffn(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, out):
+    """out (fp32) = sum_k w_k · expert_k(x) + shared(x), experts of the gated-SiLU form."""
+    if _hip(x):
+        torch.ops.dsse.moe_ffn(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, out)
+    else:
+        lref.moe_ffn(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, out)
