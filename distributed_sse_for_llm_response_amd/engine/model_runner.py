@@ -228,6 +228,7 @@ class RunnerBase:
         self.graphs = {}
         self.graph_pool = None
         self.kept_logits = None
+        self.mx_graphs = {}
 
     def _sample_commit(self, B: int) -> None:
         """Candidates per (row, vocab chunk) on each rank -> (TP: all-gather, 8 B per candidate) -> pick."""
@@ -314,6 +315,17 @@ class RunnerBase:
         self.ids.index_copy_(0, slot_idx, new_ids)
         self.ring[ring_row].index_copy_(0, slot_idx, new_ids)
         self.positions.index_copy_(0, slot_idx, last_pos + 1)
+
+    # mixed steps without captured graphs (a runner with captured mixed steps overrides these three)
+    def mixed_chunk(self, B: int) -> int:
+        """Prompt rows of a mixed step before its cost is measured."""
+        return 256
+
+    def mixed_chunks(self, B: int) -> list:
+        return []
+
+    def mixed_graph_rows(self, B: int, T: int):
+        return None
 
     def _keep_logits(self, seqs: list, x, q_start: list) -> None:
         """kept_logits [n, V] (fp32) = the logits of the rows that chunks ask for (PrefillSeq.want), in the order of

@@ -74,7 +74,9 @@ def latent_attention(h, w: dict, p: str, m: dict, eps: float):
     v = (c @ w[p + "uv"].T).view(T, H, dv)
     s = (torch.einsum("ihd,jhd->hij", q_n, k_n) + torch.einsum("ihd,jd->hij", q_r, k_r)) * float(m["scale"])
     i, j = pos[:, None], pos[None, :]
-    seen = (i - j >= 0) & (i - j < int(m["mask"]["size"]))
+    seen = i - j >= 0
+    if m.get("mask"):
+        seen = seen & (i - j < int(m["mask"]["size"]))
     s = s.masked_fill(~seen[None], float("-inf"))
     o = torch.einsum("hij,jhd->ihd", torch.softmax(s, -1), v).reshape(T, H * dv)
     return o @ w[p + "o"].T
