@@ -129,7 +129,7 @@ void embed_rows(const Tensor& ids, const Tensor& embed, Tensor& resid, Tensor& x
 }
 
 void latent_kv_write(const Tensor& ckr, const Tensor& norm_w, const Tensor& positions, const Tensor& slots,
-                     const Tensor& rope, Tensor& cache, double eps) {
+                     const Tensor& rope, Tensor& cache, double eps, const OptTensor& vt) {
   f32t(ckr, "ckr");
   gpu(norm_w, "norm_w");
   i32(positions, "positions");
@@ -154,12 +154,19 @@ void latent_kv_write(const Tensor& ckr, const Tensor& norm_w, const Tensor& posi
   p.eps = (float)eps;
   p.f32 = elem(cache, "cache");
   DSSE_CHECK_HIP(dsse_latent_kv_write(&p, cur_stream()));
+  if (vt.has_value()) {
+    gpu(*vt, "vt");
+    same(cache, *vt, "vt");
+    TORCH_CHECK(vt->dim() == 3 && vt->size(0) == cache.size(0) && vt->size(1) == rk && vt->size(2) == dsse::kBS,
+                "vt must be [pages, rk, 32]");
+    DSSE_CHECK_HIP(dsse_latent_vt_write(&p, vt->data_ptr(), cur_stream()));
+  }
 }
 
 void latent_attention(const Tensor& q, const Tensor& q_abs, const Tensor& cache, const Tensor& block_tables,
                       const Tensor& q_start, const Tensor& q_len, const Tensor& ctx_len, const Tensor& work_seq,
                       const Tensor& work_tile, const Tensor& rope, Tensor& out, int64_t window, double scale,
-                      int64_t qt) {
+                      int64_t qt, const OptTensor& vt, int64_t hp) {
   gpu(q, "q");
   f32t(q_abs, "q_abs");
   gpu(cache, "cache");
@@ -202,6 +209,17 @@ void latent_attention(const Tensor& q, const Tensor& q_abs, const Tensor& cache,
   p.rope_len = (int)rope.size(0);
   p.scale = (float)scale;
   p.f32 = elem(q, "q");
+  if (vt.has_value()) {
+    // MFMA form: work_tile counts tiles of qt rows, hp heads side by side, qt * hp = 16 columns
+    gpu(*vt, "vt");
+    TORCH_CHECK(q.scalar_type() == at::kBFloat16 && vt->scalar_type() == at::kBFloat16, "the MFMA form is bf16");
+    TORCH_CHECK(vt->dim() == 3 && vt->size(0) == cache.size(0) && vt->size(1) == rk && vt->size(2) == dsse::kBS,
+                "vt must be [pages, rk, 32]");
+    TORCH_CHECK(qt * hp == 16 && (rk == 64 || rk == 128 || rk == 256 || rk == 512) && dr % 32 == 0,
+                "the MFMA form needs qt * hp = 16, rk in {64, 128, 256, 512}, dr % 32 == 0");
+    DSSE_CHECK_HIP(dsse_latent_flash((int)work_seq.numel(), &p, vt->data_ptr(), (int)qt, (int)hp, cur_stream()));
+    return;
+  }
   DSSE_CHECK_HIP(dsse_latent_attention((int)work_seq.numel(), &p, cur_stream()));
 }
 
@@ -361,10 +379,10 @@ TORCH_LIBRARY_FRAGMENT(dsse, m) {
   m.def("scalar_norm(Tensor? y, Tensor g, Tensor(a!) resid, Tensor(b!) xb, float eps) -> ()");
   m.def("embed_rows(Tensor ids, Tensor embed, Tensor(a!) resid, Tensor(b!) xb) -> ()");
   m.def("latent_kv_write(Tensor ckr, Tensor norm_w, Tensor positions, Tensor slots, Tensor rope, Tensor(a!) cache, "
-        "float eps) -> ()");
+        "float eps, Tensor(b!)? vt=None) -> ()");
   m.def("latent_attention(Tensor q, Tensor q_abs, Tensor cache, Tensor block_tables, Tensor q_start, Tensor q_len, "
         "Tensor ctx_len, Tensor work_seq, Tensor work_tile, Tensor rope, Tensor(a!) out, int window, float scale, "
-        "int qt) -> ()");
+        "int qt, Tensor? vt=None, int hp=1) -> ()");
   m.def("conv_state(Tensor inp, Tensor taps, Tensor? bias, Tensor(a!) tail, Tensor q_start, Tensor q_len, "
         "Tensor ctx_len, Tensor state_slot, Tensor(b!) out, Tensor(c!) out_b) -> ()");
   m.def("lru_scan(Tensor u, Tensor gates, Tensor y, Tensor lam, Tensor(a!) state, Tensor q_start, Tensor q_len, "

@@ -148,6 +148,143 @@ __global__ __launch_bounds__(256) void latent_attention_rows_kernel(LatentAttnPa
 }
 
 }  // namespace
+
+// ---------------------------------------------------------------------------------------------------------------------
+// MFMA form (bf16): one wave per work item, 16 query columns, 32 keys (one cache page) per step, no LDS for keys or
+// values.  A column is a (row, head) pair: a decode step puts 16 heads of its one row side by side (the page is read
+// once for all of them), a prompt portion puts 16 rows of one head (or rt rows x hp heads).
+//
+//   S^T[key, col] = K[key, :] . Q[col, :]     A = the page's key rows straight from global memory (16 B per lane),
+//                                              B = the columns' query vectors [q_abs | rot(q_rot)] staged in LDS as bf16
+//   online softmax per column in fp32 (a column's 32 scores sit in 8 registers of its 4 lanes: rows4_max / rows4_sum)
+//   O^T[dim, col] += V^T[dim, key] . P^T[key, col]
+//                                              A = the TRANSPOSED latent page vt[page][dim][32 keys] (16 B per lane),
+//                                              B = the probabilities exactly as the score accumulators hold them
+//
+// The last step needs no shuffle because which key a (lane group g, element j) pair of the k axis stands for only has
+// to agree between A and B: the scores of lane group g are keys 4g..4g+3 of both 16-key halves, so the transposed page
+// stores key k at position 8 ((k & 15) >> 2) + 4 (k >> 4) + (k & 3) (the dense KV cache's V pages use the same order).
+template <int NT>  // rk / 16 value tiles
+__global__ __launch_bounds__(64) void latent_flash_kernel(LatentAttnParams p, const bf16* __restrict__ vt, int rt, int hp) {
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  const int D = p.rk + p.dr;
+  const int ldq = D + 8;  // bf16 elements per LDS row (16 B of padding)
+  bf16* qs = reinterpret_cast<bf16*>(smem_raw);  // [16][ldq]
+  const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
+  const int seq = p.work_seq[blockIdx.x], tile = p.work_tile[blockIdx.x];
+  const int ql = p.q_len[seq];
+  if (tile * rt >= ql) return;
+  const int q0 = p.q_start[seq], pos0 = p.ctx_len[seq] - ql;
+  // this lane's column
+  const int c_off = tile * rt + r / hp, c_head = blockIdx.y * hp + r % hp;
+  const bool c_ok = c_off < ql && c_head < p.H;
+  const int c_pos = c_ok ? pos0 + c_off : -1;
+  const int64_t c_row = q0 + (c_ok ? c_off : 0);
+  // stage the 16 query vectors: lane group g fills coordinates g, g + 4, ... (in chunks of 8) of column r
+  {
+    const float* qa = p.q_abs + (c_row * p.H + (c_ok ? c_head : 0)) * p.rk;
+    for (int d = 8 * g; d < p.rk; d += 32) {
+      bf16x8 v;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = (bf16)(c_ok ? qa[d + j] : 0.0f);
+      *reinterpret_cast<bf16x8*>(qs + r * ldq + d) = v;
+    }
+    const bf16* qr = reinterpret_cast<const bf16*>(p.q) + (c_row * p.H + (c_ok ? c_head : 0)) * (p.dn + p.dr) + p.dn;
+    const int pp = c_pos < 0 ? 0 : (c_pos >= p.rope_len ? p.rope_len - 1 : c_pos);
+    const float2* cs = p.rope + (int64_t)pp * (p.dr / 2);
+    for (int d = 8 * g; d < p.dr; d += 32) {
+      bf16x8 v;
+#pragma unroll
+      for (int j = 0; j < 8; j += 2) {
+        const float a = c_ok ? (float)qr[d + j] : 0.0f, b = c_ok ? (float)qr[d + j + 1] : 0.0f;
+        const float2 t = cs[(d + j) / 2];
+        v[j] = (bf16)(a * t.x - b * t.y);
+        v[j + 1] = (bf16)(b * t.x + a * t.y);
+      }
+      *reinterpret_cast<bf16x8*>(qs + r * ldq + p.rk + d) = v;
+    }
+  }
+  __syncthreads();
+  // key range of the tile: from the first row's window start to the last row's position
+  const int last_off = (tile * rt + rt - 1 < ql ? tile * rt + rt - 1 : ql - 1);
+  const int hi = pos0 + last_off;
+  int lo = pos0 + tile * rt - p.window + 1;
+  lo = lo > 0 ? lo : 0;
+  const int* bt = p.block_tables + (int64_t)seq * p.max_blocks;
+  const bf16* rows = reinterpret_cast<const bf16*>(p.cache);
+  f32x4 O[NT];
+#pragma unroll
+  for (int n = 0; n < NT; ++n) O[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int nks = D / 32;
+  for (int pg = lo / kBS; pg <= hi / kBS; ++pg) {
+    int blk = bt[pg];
+    blk = (unsigned)blk < (unsigned)p.num_blocks ? blk : 0;
+    const bf16* krow0 = rows + ((int64_t)blk * kBS + r) * D + 8 * g;        // key r of the page's first half
+    const bf16* krow1 = krow0 + (int64_t)16 * D;                             // key 16 + r
+    f32x4 s0 = f32x4{0.f, 0.f, 0.f, 0.f}, s1 = s0;
+    for (int s = 0; s < nks; ++s) {
+      const bf16x8 b = *reinterpret_cast<const bf16x8*>(qs + r * ldq + 32 * s + 8 * g);
+      s0 = mfma16x16x32(ld_bf16x8(krow0 + 32 * s), b, s0);
+      s1 = mfma16x16x32(ld_bf16x8(krow1 + 32 * s), b, s1);
+    }
+    // lane (r, g): column r, keys pg * 32 + 4 g + i (s0) and + 16 (s1)
+    float sv[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int key = pg * kBS + (i < 4 ? 4 * g + i : 16 + 4 * g + (i - 4));
+      const bool seen = c_ok && key <= c_pos && c_pos - key < p.window;
+      sv[i] = seen ? (i < 4 ? s0[i] : s1[i - 4]) * p.scale : -INFINITY;
+      mx = fmaxf(mx, sv[i]);
+    }
+    mx = rows4_max(mx);
+    const float mn = fmaxf(m, mx);
+    const float corr = mn == -INFINITY ? 1.0f : expf(m - mn);  // m = -inf, mn finite: exp(-inf) = 0
+    bf16x8 pf;
+    float ps = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float e = sv[i] == -INFINITY ? 0.0f : expf(sv[i] - mn);
+      ps += e;
+      pf[i] = (bf16)e;
+    }
+    l = l * corr + rows4_sum(ps);
+    m = mn;
+    const bf16* vrow = vt + ((int64_t)blk * p.rk + r) * kBS + 8 * g;  // dim r of value tile 0, positions 8g..8g+7
+#pragma unroll
+    for (int n = 0; n < NT; ++n) {
+      f32x4 o = O[n];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] *= corr;
+      O[n] = mfma16x16x32(ld_bf16x8(vrow + (int64_t)n * 16 * kBS), pf, o);
+    }
+  }
+  if (c_ok) {
+    bf16* out = reinterpret_cast<bf16*>(p.out) + (c_row * p.H + c_head) * p.rk;
+    const float inv = l > 0.f ? 1.0f / l : 0.0f;
+#pragma unroll
+    for (int n = 0; n < NT; ++n) {
+      bf16x4 v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = (bf16)(O[n][i] * inv);
+      *reinterpret_cast<bf16x4*>(out + 16 * n + 4 * g) = v;
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void latent_vt_write_kernel(LatentKvWriteParams p, T* __restrict__ vt) {
+  // after latent_kv_write: copy the token's normed latent from its cache row into the transposed page
+  const int row = blockIdx.x;
+  const int slot = p.slots[row];
+  if (slot < 0 || slot >= p.num_slots) return;
+  const int blk = slot / kBS, off = slot % kBS;
+  const int at = ((off & 15) >> 2) * 8 + ((off >> 4) & 1) * 4 + (off & 3);
+  const T* src = reinterpret_cast<const T*>(p.cache) + (int64_t)slot * (p.rk + p.dr);
+  for (int d = threadIdx.x; d < p.rk; d += blockDim.x) vt[((int64_t)blk * p.rk + d) * kBS + at] = src[d];
+}
+
 }  // namespace dsse
 
 extern "C" hipError_t dsse_latent_kv_write(const dsse::LatentKvWriteParams* p, hipStream_t st) {
@@ -164,5 +301,32 @@ extern "C" hipError_t dsse_latent_attention(int num_work, const dsse::LatentAttn
   dim3 grid(num_work, p->H);
   if (p->f32) hipLaunchKernelGGL(dsse::latent_attention_rows_kernel<float>, grid, dim3(256), lds, st, *p);
   else hipLaunchKernelGGL(dsse::latent_attention_rows_kernel<bf16>, grid, dim3(256), lds, st, *p);
+  return hipGetLastError();
+}
+
+extern "C" hipError_t dsse_latent_vt_write(const dsse::LatentKvWriteParams* p, void* vt, hipStream_t st) {
+  if (p->T <= 0) return hipSuccess;
+  if (p->f32)
+    hipLaunchKernelGGL(dsse::latent_vt_write_kernel<float>, dim3(p->T), dim3(256), 0, st, *p, reinterpret_cast<float*>(vt));
+  else
+    hipLaunchKernelGGL(dsse::latent_vt_write_kernel<bf16>, dim3(p->T), dim3(256), 0, st, *p, reinterpret_cast<bf16*>(vt));
+  return hipGetLastError();
+}
+
+// rt rows x hp heads = 16 columns per work item; work_tile counts tiles of rt rows
+extern "C" hipError_t dsse_latent_flash(int num_work, const dsse::LatentAttnParams* p, const void* vt, int rt, int hp,
+                                        hipStream_t st) {
+  if (num_work <= 0) return hipSuccess;
+  if (p->f32 || rt * hp != 16 || p->rk % 32 || p->dr % 32) return hipErrorInvalidValue;
+  const size_t lds = 16 * (size_t)(p->rk + p->dr + 8) * sizeof(bf16);
+  dim3 grid(num_work, (p->H + hp - 1) / hp);
+  const bf16* v = reinterpret_cast<const bf16*>(vt);
+  switch (p->rk / 16) {
+    case 4: hipLaunchKernelGGL(dsse::latent_flash_kernel<4>, grid, dim3(64), lds, st, *p, v, rt, hp); break;
+    case 8: hipLaunchKernelGGL(dsse::latent_flash_kernel<8>, grid, dim3(64), lds, st, *p, v, rt, hp); break;
+    case 16: hipLaunchKernelGGL(dsse::latent_flash_kernel<16>, grid, dim3(64), lds, st, *p, v, rt, hp); break;
+    case 32: hipLaunchKernelGGL(dsse::latent_flash_kernel<32>, grid, dim3(64), lds, st, *p, v, rt, hp); break;
+    default: return hipErrorInvalidValue;
+  }
   return hipGetLastError();
 }

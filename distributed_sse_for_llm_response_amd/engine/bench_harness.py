@@ -104,7 +104,11 @@ class PacedStubEngine:
 def _build_runner(model: str, device, streams: int, prompt_len: int, total_steps: int, tp: int, use_graphs: bool,
                   rank: int, world: int, comm: TPComm | None = None):
     # on CPU the 7B architecture is replaced by the tiny one (plumbing runs); named small configs are kept
-    cfg = get_config(model) if device.type == "cuda" or not model.startswith("mistral-7b") else TINY
+    from ..models import registry
+
+    fam, cfg, ckpt = registry.resolve(model)
+    if fam.name == "mistral" and device.type != "cuda" and model.startswith("mistral-7b"):
+        cfg = TINY
     if comm is None:
         comm = TPComm()
         if tp > 1:
@@ -112,11 +116,11 @@ def _build_runner(model: str, device, streams: int, prompt_len: int, total_steps
 
             grp, _ = make_groups(world, tp)
             comm = TPComm(rank=rank % tp, size=tp, group=grp)
-    w = random_engine_weights(cfg, tp_rank=comm.rank, tp_size=comm.size, device=device, seed=1234)
+    w = registry.load_weights(fam, cfg, ckpt, device=device, seed=1234, tp_rank=comm.rank, tp_size=comm.size)
     max_len = prompt_len + total_steps + 2 * PAGE
     nblk = streams * (blocks_needed(max_len) + 1) + 4
-    runner = ModelRunner(w, num_blocks=nblk, max_batch=streams, max_model_len=max_len, device=device, comm=comm,
-                         use_graphs=use_graphs)
+    runner = registry.make_runner(fam, w, num_blocks=nblk, max_batch=streams, max_model_len=max_len, device=device,
+                                  comm=comm, use_graphs=use_graphs)
     return cfg, runner
 
 

@@ -66,9 +66,14 @@ class LatentKVCache:
     allocator and the block tables are the ones the dense KV cache uses.  ``widths`` maps layer index -> rank + rot
     (layers without attention have no entry)."""
 
-    def __init__(self, widths: dict, num_blocks: int, device, dtype=torch.bfloat16):
+    def __init__(self, widths: dict, num_blocks: int, device, dtype=torch.bfloat16, transposed: dict | None = None):
         self.num_blocks = num_blocks
         self.layers = {li: torch.zeros(num_blocks, PAGE, w, device=device, dtype=dtype) for li, w in widths.items()}
+        # layers on the MFMA attention form also keep the latent in transposed pages [blocks, rank, PAGE] (tokens
+        # permuted inside a page, ops/layers_reference.py vt_position): its value operand is then one 16-byte load per
+        # lane, as with the dense cache's V pages.  `transposed` maps layer index -> rank for those layers.
+        self.vt = {li: torch.zeros(num_blocks, rk, PAGE, device=device, dtype=dtype)
+                   for li, rk in (transposed or {}).items()}
 
     def __getitem__(self, li: int) -> torch.Tensor:
         return self.layers[li]

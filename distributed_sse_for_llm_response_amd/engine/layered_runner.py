@@ -35,6 +35,7 @@ from .model_runner import RunnerBase, _capture, batch_buckets
 from .weights import LayeredWeights
 
 ATTN_ROWS_TILE = 4    # query rows per work item of the row-wise attention kernel (prompt portions)
+FLASH_ROWS_TILE = 16  # query rows per work item of the MFMA attention form (x 16 / rows heads = 16 columns)
 
 
 class LayeredRunner(RunnerBase):
@@ -55,7 +56,9 @@ class LayeredRunner(RunnerBase):
         self._init_slots(max_batch, self.max_blocks, cfg.vocab_size, dev, self.comm)
         att = {i: L.mixer for i, L in enumerate(cfg.layers) if L.kind == "latent_attention"}
         rec = {i: L.mixer for i, L in enumerate(cfg.layers) if L.kind == "rglru"}
-        self.kv = LatentKVCache({i: m.kv_rank + m.rot_dim for i, m in att.items()}, num_blocks, dev, self.dtype)
+        flash = {i: m.kv_rank for i, m in att.items() if ops.latent_flash_ok(self.dtype, m.kv_rank, m.rot_dim)}
+        self.kv = LatentKVCache({i: m.kv_rank + m.rot_dim for i, m in att.items()}, num_blocks, dev, self.dtype,
+                                transposed=flash)
         self.state = RecurrentStateCache({i: (m.width, m.conv) for i, m in rec.items()}, max_batch, dev)
         # one rotation table per distinct (rotation, rotated width)
         self._rope = {}
@@ -104,11 +107,18 @@ class LayeredRunner(RunnerBase):
         attn = d["attn"][:M * H * dv].view(M, H, dv)
         ops.gemm_rm(d["xb"], Lw.q, q.view(M, H * (dn + dr)))
         ops.gemm_rm(d["xb"], Lw.dkv, ckr)
-        ops.latent_kv_write(ckr, Lw.dkv_norm, pos, slots, rope, cache, self.cfg.eps)
+        vt = self.kv.vt.get(li)
+        ops.latent_kv_write(ckr, Lw.dkv_norm, pos, slots, rope, cache, self.cfg.eps, vt)
         ops.gemm_rm(q[:, :, :dn].permute(1, 0, 2), Lw.uk_t, qabs.permute(1, 0, 2))
         for g in groups:
-            ops.latent_attention(q, qabs, cache, g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"], g["wt"], rope, lat,
-                                 m.window, m.scale, g["qt"])
+            if vt is not None:  # MFMA form: a decode row's heads side by side, a portion's rows in tiles of 16
+                dec = g["qt"] == 1
+                ops.latent_attention(q, qabs, cache, g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"] if dec else g["fs"],
+                                     g["wt"] if dec else g["ft"], rope, lat, m.window, m.scale,
+                                     1 if dec else FLASH_ROWS_TILE, vt, 16 if dec else 16 // FLASH_ROWS_TILE)
+            else:
+                ops.latent_attention(q, qabs, cache, g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"], g["wt"], rope, lat,
+                                     m.window, m.scale, g["qt"])
         ops.gemm_rm(lat.permute(1, 0, 2), Lw.uv, attn.permute(1, 0, 2))
         ops.gemm_rm(attn.view(M, H * dv), Lw.o, d["y"])
 
@@ -220,7 +230,7 @@ class LayeredRunner(RunnerBase):
         """Packed metadata of prompt portions whose rows start at `row0`: one pinned upload.  Returns (T, q_start
         list, device dict: ids / pos / slots per row, qs / ql / ctx / ss per sequence, ws / wt work items, bt)."""
         n = len(seqs)
-        ids_l, pos_l, slots_l, qs, ql, ctx, ss, ws, wt = [], [], [], [], [], [], [], [], []
+        ids_l, pos_l, slots_l, qs, ql, ctx, ss, ws, wt, fs, ft = [], [], [], [], [], [], [], [], [], [], []
         bt = torch.zeros(n, self.max_blocks, dtype=torch.int32)
         row = 0
         for i, s in enumerate(seqs):
@@ -238,16 +248,19 @@ class LayeredRunner(RunnerBase):
             nt = math.ceil(m / ATTN_ROWS_TILE)
             ws += [i] * nt
             wt += list(range(nt))
+            nf = math.ceil(m / FLASH_ROWS_TILE)
+            fs += [i] * nf
+            ft += list(range(nf))
             row += m
         T = row
-        meta = torch.from_numpy(np.concatenate(ids_l + pos_l + slots_l + [np.asarray(qs + ql + ctx + ss + ws + wt,
+        meta = torch.from_numpy(np.concatenate(ids_l + pos_l + slots_l + [np.asarray(qs + ql + ctx + ss + ws + wt + fs + ft,
                                                                                      dtype=np.int64)]).astype(np.int32))
         if self.device.type == "cuda":
             meta = meta.pin_memory().to(self.device, non_blocking=True)
             bt = bt.pin_memory().to(self.device, non_blocking=True)
         d, o = {}, 0
         for name, k in (("ids", T), ("pos", T), ("slots", T), ("qs", n), ("ql", n), ("ctx", n), ("ss", n),
-                        ("ws", len(ws)), ("wt", len(ws))):
+                        ("ws", len(ws)), ("wt", len(ws)), ("fs", len(fs)), ("ft", len(fs))):
             d[name], o = meta[o:o + k], o + k
         d["bt"] = bt
         d["qt"] = ATTN_ROWS_TILE

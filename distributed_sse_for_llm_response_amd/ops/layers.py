@@ -45,23 +45,31 @@ def embed_rows(ids, embed, resid, xb):
         lref.embed_rows(ids, embed, resid, xb)
 
 
-def latent_kv_write(ckr, norm_w, positions, slots, rope, cache, eps: float):
-    """cache[slot] = [rms-norm(ckr[:, :rk]) · norm_w | rot(ckr[:, rk:])] for rows with slot >= 0."""
+def latent_kv_write(ckr, norm_w, positions, slots, rope, cache, eps: float, vt=None):
+    """cache[slot] = [rms-norm(ckr[:, :rk]) · norm_w | rot(ckr[:, rk:])] for rows with slot >= 0; vt (optional,
+    [pages, rk, 32]) receives the latent once more in transposed pages (the MFMA attention's value operand)."""
     if _hip(ckr):
-        torch.ops.dsse.latent_kv_write(ckr, norm_w, positions, slots, rope, cache, eps)
+        torch.ops.dsse.latent_kv_write(ckr, norm_w, positions, slots, rope, cache, eps, vt)
     else:
-        lref.latent_kv_write(ckr, norm_w, positions, slots, rope, cache, eps)
+        lref.latent_kv_write(ckr, norm_w, positions, slots, rope, cache, eps, vt)
+
+
+def latent_flash_ok(dtype, rk: int, dr: int) -> bool:
+    """Shapes the MFMA form of latent_attention covers (everything else takes the row kernel)."""
+    return dtype == torch.bfloat16 and rk in (64, 128, 256, 512) and dr % 32 == 0
 
 
 def latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile, rope, out,
-                     window: int, scale: float, qt: int):
-    """Sliding-window multi-query attention over the latent cache (folded form), `qt` query rows per work item."""
+                     window: int, scale: float, qt: int, vt=None, hp: int = 1):
+    """Sliding-window multi-query attention over the latent cache (folded form), `qt` query rows per work item.
+    With vt (transposed latent pages, latent_flash_ok shapes): the MFMA form, qt rows x hp heads = 16 columns per
+    item; without: the row kernel (any sizes, both element types)."""
     if _hip(q):
         torch.ops.dsse.latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile,
-                                        rope, out, window, scale, qt)
+                                        rope, out, window, scale, qt, vt, hp)
     else:
         lref.latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile, rope, out,
-                              window, scale, qt)
+                              window, scale, qt, vt)
 
 
 def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b):

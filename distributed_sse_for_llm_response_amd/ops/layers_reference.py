@@ -55,7 +55,12 @@ def _rotate(v, cs):
     return out
 
 
-def latent_kv_write(ckr, norm_w, positions, slots, rope, cache, eps):
+def vt_position(off):
+    """Place of token `off` (0..31) inside a transposed latent page (the MFMA attention's key order)."""
+    return ((off & 15) >> 2) * 8 + ((off >> 4) & 1) * 4 + (off & 3)
+
+
+def latent_kv_write(ckr, norm_w, positions, slots, rope, cache, eps, vt=None):
     T, rk = ckr.shape[0], norm_w.numel()
     flat = cache.view(-1, cache.shape[-1])
     c = ckr[:, :rk]
@@ -66,10 +71,14 @@ def latent_kv_write(ckr, norm_w, positions, slots, rope, cache, eps):
     sl = slots[:T].long()
     ok = (sl >= 0) & (sl < flat.shape[0])
     flat[sl[ok]] = row[ok]
+    if vt is not None:
+        good = sl[ok]
+        vt[good // PAGE, :, vt_position(good % PAGE)] = row[ok][:, :rk]
 
 
 def latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile, rope, out, window,
-                     scale, qt):
+                     scale, qt, vt=None):
+    """With vt the values come from the transposed pages (the same numbers in another place), so a wrong place shows."""
     rk = q_abs.shape[2]
     dr = cache.shape[2] - rk
     dn = q.shape[2] - dr
@@ -91,7 +100,8 @@ def latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, wor
             qr = _rotate(q[row, :, dn:].float(), rope[min(max(pos, 0), rope.shape[0] - 1)])
             sc = (q_abs[row].float() @ kv[:, :rk].t() + qr @ kv[:, rk:].t()) * scale
             p = torch.softmax(sc, dim=-1)
-            out[row] = (p @ kv[:, :rk]).to(out.dtype)
+            val = kv[:, :rk] if vt is None else vt[rows // PAGE, :, vt_position(rows % PAGE)].float()
+            out[row] = (p @ val).to(out.dtype)
 
 
 def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b):

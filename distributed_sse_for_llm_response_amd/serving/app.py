@@ -21,7 +21,6 @@ import torch
 
 from .. import runtime as rt_mod
 from ..engine.engine import FINISH_CODES, EngineFault, LLMEngine, SamplingParams, TokenEvent
-from ..engine.kv_cache import KVCache
 from ..engine.model_runner import ModelRunner
 from ..models.mistral import TINY, get_config, init_standard_weights
 from ..models.tokenizer import get_tokenizer, prompt_for_request
@@ -30,30 +29,30 @@ from .faults import FaultPlan, StepTracer, Watchdog
 
 
 def build_engine(cfg: ServeConfig, device=None, comm=None):
-    """Weights + KV cache + runner + engine for this process (one DP replica / TP rank)."""
-    from ..engine.weights import convert_standard, load_safetensors, random_engine_weights
+    """Weights + KV cache + runner + engine for this process (one DP replica / TP rank).  ``cfg.model`` is a
+    configuration name or a checkpoint directory; the registry (models/registry.py) picks the family, its weight
+    loader and its runner."""
+    from ..models import registry
 
+    fam, mcfg, ckpt = registry.resolve(cfg.model)
+    tp_rank, tp = (comm.rank, comm.size) if comm is not None else (0, 1)
+    path = cfg.weights_path or ckpt
     if cfg.engine == "cpu":
-        mcfg = TINY if cfg.model.startswith("mistral-7b") else get_config(cfg.model)
-        tp_rank, tp = (comm.rank, comm.size) if comm is not None else (0, 1)
-        w = convert_standard(mcfg, init_standard_weights(mcfg, seed=cfg.seed), tp_rank=tp_rank, tp_size=tp)
-        runner = ModelRunner(w, num_blocks=256, max_batch=min(cfg.max_batch, 8),
-                             max_model_len=min(cfg.max_model_len, 1024), device="cpu", comm=comm, use_graphs=False)
+        if fam.name == "mistral" and cfg.model.startswith("mistral-7b"):
+            mcfg = TINY
+        w = registry.load_weights(fam, mcfg, path, device="cpu", seed=cfg.seed, tp_rank=tp_rank, tp_size=tp)
+        runner = registry.make_runner(fam, w, num_blocks=256, max_batch=min(cfg.max_batch, 8),
+                                      max_model_len=min(cfg.max_model_len, 1024), device="cpu", comm=comm,
+                                      use_graphs=False)
     else:
         device = device or torch.device("cuda", torch.cuda.current_device())
-        mcfg = get_config(cfg.model)
-        tp_rank, tp = (comm.rank, comm.size) if comm is not None else (0, 1)
-        if cfg.weights_path:
-            w = load_safetensors(mcfg, cfg.weights_path, tp_rank, tp, device)
-        else:
-            w = random_engine_weights(mcfg, tp_rank=tp_rank, tp_size=tp, device=device, seed=cfg.seed)
+        w = registry.load_weights(fam, mcfg, path, device=device, seed=cfg.seed, tp_rank=tp_rank, tp_size=tp)
         free, total = torch.cuda.mem_get_info(device)
         budget = int(total * cfg.gpu_memory_utilization) - (total - free) - (2 << 30)
-        nkv = mcfg.num_kv_heads // tp
-        nblk = max(64, min(KVCache.blocks_for_budget(budget, mcfg.num_layers, nkv),
+        nblk = max(64, min(registry.cache_blocks_for_budget(mcfg, budget, tp),
                            cfg.max_batch * (cfg.max_model_len // 32 + 2) * 4))
-        runner = ModelRunner(w, num_blocks=nblk, max_batch=cfg.max_batch, max_model_len=cfg.max_model_len,
-                             device=device, comm=comm)
+        runner = registry.make_runner(fam, w, num_blocks=nblk, max_batch=cfg.max_batch,
+                                      max_model_len=cfg.max_model_len, device=device, comm=comm)
         runner.capture()
     tok = get_tokenizer(mcfg.vocab_size, cfg.tokenizer_path or None)
     engine = LLMEngine(runner, eos_id=tok.eos_id, prefill_budget=cfg.prefill_budget, max_pause_s=cfg.max_pause_s,

@@ -1,0 +1,88 @@
+"""The MFMA form of latent attention against the row kernel and the PyTorch reference of the same op, on the same
+bf16 inputs: random block tables, several sequences with unequal portions, windows that end inside, at and across
+pages, decode columns (a row's heads side by side, also more than 16 heads) and prompt tiles."""
+import math
+
+import pytest
+import torch
+
+from distributed_sse_for_llm_response_amd import ops
+from distributed_sse_for_llm_response_amd.ops import layers_reference as lref
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(gpu, H, dn, dr, rk, window, seqs, qt_rows, seed):
+    """seqs: [(context before the step, rows in the step)].  Returns the three outputs [T, H, rk]."""
+    g = torch.Generator().manual_seed(seed)
+    D = rk + dr
+    total = sum(c + n for c, n in seqs)
+    pages = sum(math.ceil((c + n) / 32) for c, n in seqs) + 3
+    perm = torch.randperm(pages, generator=g).tolist()
+    mb = max(math.ceil((c + n) / 32) for c, n in seqs) + 1
+    bt = torch.zeros(len(seqs), mb, dtype=torch.int32)
+    cache = torch.zeros(pages, 32, D, dtype=torch.bfloat16)
+    vt = torch.zeros(pages, rk, 32, dtype=torch.bfloat16)
+    rope = torch.zeros(max(c + n for c, n in seqs) + 1, dr // 2, 2)
+    ang = torch.arange(rope.shape[0])[:, None] * (100.0 ** (-torch.arange(dr // 2) / (dr // 2)))[None, :]
+    rope[..., 0], rope[..., 1] = ang.cos() * 1.1, ang.sin() * 1.1
+    qs, ql, ctx, ws, wt, fs, ft = [], [], [], [], [], [], []
+    T = sum(n for _, n in seqs)
+    ckr = torch.randn(total, D, generator=g) * 1.5
+    norm_w = (1.0 + 0.1 * torch.randn(rk, generator=g)).to(torch.bfloat16)
+    pos, slots, at, row = [], [], 0, 0
+    for i, (c, n) in enumerate(seqs):
+        npg = math.ceil((c + n) / 32)
+        mine, perm = perm[:npg], perm[npg:]
+        bt[i, :npg] = torch.tensor(mine, dtype=torch.int32)
+        for p in range(c + n):
+            pos.append(p)
+            slots.append(mine[p // 32] * 32 + p % 32)
+        qs.append(row), ql.append(n), ctx.append(c + n)
+        nt = math.ceil(n / qt_rows)
+        ws += [i] * nt
+        wt += list(range(nt))
+        row += n
+        at += c + n
+    q = (torch.randn(T, H, dn + dr, generator=g) * 2.0).to(torch.bfloat16)
+    q_abs = torch.randn(T, H, rk, generator=g) * 2.0
+    dev = dict(device=gpu)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, **dev)  # noqa: E731
+    cache_g, vt_g = cache.to(gpu), vt.to(gpu)
+    ops.latent_kv_write(ckr.to(gpu), norm_w.to(gpu), i32(pos), i32(slots), rope.to(gpu), cache_g, 1e-5, vt_g)
+    lref.latent_kv_write(ckr, norm_w, torch.tensor(pos, dtype=torch.int32), torch.tensor(slots, dtype=torch.int32), rope,
+                         cache, 1e-5, vt)
+    assert torch.equal(cache_g.cpu(), cache) or torch.allclose(cache_g.cpu().float(), cache.float(), atol=2e-2, rtol=2e-2)
+    assert torch.allclose(vt_g.cpu().float(), vt.float(), atol=2e-2, rtol=2e-2)
+    scale = 0.5 / math.sqrt(dn + dr)
+    args = (bt.to(gpu), i32(qs), i32(ql), i32(ctx))
+    out_rows = torch.zeros(T, H, rk, dtype=torch.bfloat16, **dev)
+    ops.latent_attention(q.to(gpu), q_abs.to(gpu), cache_g, *args, i32(ws), i32(wt), rope.to(gpu), out_rows, window, scale,
+                         qt_rows)
+    out_flash = torch.zeros_like(out_rows)
+    hp = 16 // qt_rows if qt_rows in (1, 2, 4, 8, 16) else 1
+    if qt_rows * hp == 16:
+        ops.latent_attention(q.to(gpu), q_abs.to(gpu), cache_g, *args, i32(ws), i32(wt), rope.to(gpu), out_flash, window,
+                             scale, qt_rows, vt_g, hp)
+    out_ref = torch.zeros(T, H, rk, dtype=torch.float32)
+    lref.latent_attention(q, q_abs, cache_g.cpu(), bt, torch.tensor(qs), torch.tensor(ql), torch.tensor(ctx),
+                          torch.tensor(ws), torch.tensor(wt), rope, out_ref, window, scale, qt_rows, vt_g.cpu())
+    return out_rows.float().cpu(), out_flash.float().cpu(), out_ref
+
+
+@pytest.mark.parametrize("H,dn,dr,rk", [(3, 16, 32, 64), (8, 32, 32, 128), (20, 8, 64, 256), (16, 24, 32, 512)])
+@pytest.mark.parametrize("window", [1, 5, 32, 33, 70, 10 ** 6])
+def test_prompt_tiles(gpu, H, dn, dr, rk, window):
+    seqs = [(0, 50), (37, 3), (64, 31), (5, 1), (90, 40)]
+    rows, flash, ref = _case(gpu, H, dn, dr, rk, window, seqs, 16, seed=H + window)
+    assert torch.allclose(rows, ref, atol=3e-2, rtol=3e-2)
+    assert torch.allclose(flash, ref, atol=5e-2, rtol=5e-2), float((flash - ref).abs().max())
+
+
+@pytest.mark.parametrize("H,dn,dr,rk", [(3, 16, 32, 64), (8, 32, 32, 128), (20, 8, 64, 256), (33, 24, 32, 512)])
+@pytest.mark.parametrize("window", [1, 2, 31, 32, 33, 64, 65, 10 ** 6])
+def test_decode_columns(gpu, H, dn, dr, rk, window):
+    seqs = [(0, 1), (31, 1), (32, 1), (33, 1), (63, 1), (64, 1), (130, 1), (7, 0), (95, 1)]
+    rows, flash, ref = _case(gpu, H, dn, dr, rk, window, seqs, 1, seed=7 * H + window)
+    assert torch.allclose(rows, ref, atol=3e-2, rtol=3e-2)
+    assert torch.allclose(flash, ref, atol=5e-2, rtol=5e-2), float((flash - ref).abs().max())
