@@ -26,7 +26,8 @@ struct GemmRmParams {
 };
 
 struct ScalarNormParams {
-  const float* y;    // [M, W] sublayer output (mode 0) -- unused in mode 1
+  const float* y;    // [M * nsum, W] sublayer output, a row's nsum consecutive parts are summed (mode 0) -- unused in mode 1
+  int nsum;
   const void* g;     // one number, element type
   float* resid;      // [M, W] fp32 stream
   void* xb;          // [M, W] element type: the stream's rounding (mode 0) / the normed stream (mode 1)
@@ -122,6 +123,26 @@ struct MoeFfnParams {
   int f32;
 };
 
+struct MoeGroupedParams {
+  const void* x;         // [M, W]
+  const int* topk_idx;   // [M, top]
+  const float* topk_w;   // [M, top]
+  const void* gate;      // [E, F, W]
+  const void* up;
+  const void* down;      // [E, W, F]
+  const void* sgate;     // shared expert (slot `top`, expert index E) or null
+  const void* sup;
+  const void* sdown;
+  int* sorted;           // [max_tiles * 16] ids (row * S + slot) grouped by expert, -1 = pad
+  int* tile_expert;      // [max_tiles]
+  int* num_tiles;        // [1]
+  void* h;               // [M * S, ldh] element type
+  float* o;              // [M * S, W]
+  int M, W, F, Fs, E, top, S, ldh, max_tiles;
+  int vec_w, vec_h;      // 16-byte fragment loads allowed on rows W wide / on rows of h
+  int f32;
+};
+
 }  // namespace dsse
 
 extern "C" {
@@ -140,4 +161,5 @@ hipError_t dsse_conv_state(const dsse::ConvStateParams* p, hipStream_t st);
 hipError_t dsse_lru_scan(const dsse::LruScanParams* p, hipStream_t st);
 hipError_t dsse_moe_router(const dsse::MoeRouterParams* p, hipStream_t st);
 hipError_t dsse_moe_ffn(const dsse::MoeFfnParams* p, hipStream_t st);
+hipError_t dsse_moe_grouped(const dsse::MoeGroupedParams* p, hipStream_t st);
 }

@@ -94,7 +94,7 @@ void gemm_rm(const Tensor& x, const Tensor& w, Tensor& out, const OptTensor& bia
   DSSE_CHECK_HIP(dsse_gemm_rm(&p, cur_stream()));
 }
 
-void scalar_norm(const OptTensor& y, const Tensor& g, Tensor& resid, Tensor& xb, double eps) {
+void scalar_norm(const OptTensor& y, const Tensor& g, Tensor& resid, Tensor& xb, double eps, int64_t nsum) {
   f32t(resid, "resid");
   gpu(xb, "xb");
   gpu(g, "g");
@@ -103,8 +103,10 @@ void scalar_norm(const OptTensor& y, const Tensor& g, Tensor& resid, Tensor& xb,
   dsse::ScalarNormParams p{};
   if (y.has_value()) {
     f32t(*y, "y");
-    TORCH_CHECK(y->sizes() == resid.sizes(), "y must match resid");
+    TORCH_CHECK(nsum >= 1 && y->dim() == 2 && y->size(0) == resid.size(0) * nsum && y->size(1) == resid.size(1),
+                "y must be [M * nsum, W]");
     p.y = y->data_ptr<float>();
+    p.nsum = (int)nsum;
   }
   p.mode = y.has_value() ? 0 : 1;
   p.g = g.data_ptr();
@@ -372,11 +374,85 @@ void moe_ffn(const Tensor& x, const Tensor& topk_idx, const Tensor& topk_w, cons
   DSSE_CHECK_HIP(dsse_moe_ffn(&p, cur_stream()));
 }
 
+// Grouped form of the routed experts: o [M * S, W] (fp32) = per-(row, slot) expert outputs times their weights, S = top
+// (+ 1 with a shared expert); the caller sums a row's S parts (scalar_norm nsum).  Scratch: sorted [tiles * 16],
+// tile_expert [tiles], num_tiles [1] (int32), h [M * S, ldh] (element type), tiles >= ceil(M S / 16) + experts.
+void moe_grouped(const Tensor& x, const Tensor& topk_idx, const Tensor& topk_w, const Tensor& gate, const Tensor& up,
+                 const Tensor& down, const OptTensor& sgate, const OptTensor& sup, const OptTensor& sdown, Tensor& sorted,
+                 Tensor& tile_expert, Tensor& num_tiles, Tensor& h, Tensor& o) {
+  gpu(x, "x");
+  i32(topk_idx, "topk_idx");
+  f32t(topk_w, "topk_w");
+  gpu(gate, "gate");
+  gpu(up, "up");
+  gpu(down, "down");
+  i32(sorted, "sorted");
+  i32(tile_expert, "tile_expert");
+  i32(num_tiles, "num_tiles");
+  gpu(h, "h");
+  f32t(o, "o");
+  same(x, gate, "gate");
+  same(x, up, "up");
+  same(x, down, "down");
+  same(x, h, "h");
+  dsse::MoeGroupedParams p{};
+  p.M = (int)x.size(0), p.W = (int)x.size(1);
+  TORCH_CHECK(x.dim() == 2 && gate.dim() == 3 && gate.size(2) == p.W && up.sizes() == gate.sizes(), "gate / up must be [E, F, W]");
+  p.E = (int)gate.size(0), p.F = (int)gate.size(1), p.top = (int)topk_idx.size(1);
+  TORCH_CHECK(down.dim() == 3 && down.size(0) == p.E && down.size(1) == p.W && down.size(2) == p.F, "down must be [E, W, F]");
+  TORCH_CHECK(topk_idx.dim() == 2 && topk_idx.size(0) == p.M && topk_w.sizes() == topk_idx.sizes(), "routing shapes");
+  p.S = p.top;
+  if (sgate.has_value()) {
+    TORCH_CHECK(sup.has_value() && sdown.has_value(), "the shared expert needs gate, up and down");
+    gpu(*sgate, "sgate");
+    gpu(*sup, "sup");
+    gpu(*sdown, "sdown");
+    same(x, *sgate, "sgate");
+    same(x, *sup, "sup");
+    same(x, *sdown, "sdown");
+    p.Fs = (int)sgate->size(0);
+    TORCH_CHECK(sgate->dim() == 2 && sgate->size(1) == p.W && sup->sizes() == sgate->sizes() && sdown->dim() == 2 &&
+                    sdown->size(0) == p.W && sdown->size(1) == p.Fs,
+                "shared expert shapes");
+    p.sgate = sgate->data_ptr();
+    p.sup = sup->data_ptr();
+    p.sdown = sdown->data_ptr();
+    p.S = p.top + 1;
+  }
+  const int64_t ids = (int64_t)p.M * p.S;
+  p.max_tiles = (int)tile_expert.numel();
+  TORCH_CHECK(p.max_tiles >= (ids + 15) / 16 + p.E + 1 && sorted.numel() >= (int64_t)p.max_tiles * 16 && p.max_tiles <= 65535,
+              "moe_grouped: scratch too small for ", ids, " ids");
+  TORCH_CHECK(h.dim() == 2 && h.size(0) >= ids && h.size(1) >= std::max(p.F, p.Fs) && o.dim() == 2 && o.size(0) == ids &&
+                  o.size(1) == p.W && p.E + 1 <= 4096,
+              "moe_grouped: h / o shapes");
+  p.ldh = (int)h.size(1);
+  p.x = x.data_ptr();
+  p.topk_idx = topk_idx.data_ptr<int>();
+  p.topk_w = topk_w.data_ptr<float>();
+  p.gate = gate.data_ptr();
+  p.up = up.data_ptr();
+  p.down = down.data_ptr();
+  p.sorted = sorted.data_ptr<int>();
+  p.tile_expert = tile_expert.data_ptr<int>();
+  p.num_tiles = num_tiles.data_ptr<int>();
+  p.h = h.data_ptr();
+  p.o = o.data_ptr<float>();
+  p.f32 = elem(x, "x");
+  const int per = p.f32 ? 4 : 8;
+  p.vec_w = p.W % per == 0;
+  p.vec_h = p.ldh % per == 0 && p.F % per == 0;
+  DSSE_CHECK_HIP(dsse_moe_grouped(&p, cur_stream()));
+}
+
 }  // namespace
 
 TORCH_LIBRARY_FRAGMENT(dsse, m) {
   m.def("gemm_rm(Tensor x, Tensor w, Tensor(a!) out, Tensor? bias=None, int act=0) -> ()");
-  m.def("scalar_norm(Tensor? y, Tensor g, Tensor(a!) resid, Tensor(b!) xb, float eps) -> ()");
+  m.def("scalar_norm(Tensor? y, Tensor g, Tensor(a!) resid, Tensor(b!) xb, float eps, int nsum=1) -> ()");
+  m.def("moe_grouped(Tensor x, Tensor topk_idx, Tensor topk_w, Tensor gate, Tensor up, Tensor down, Tensor? sgate, "
+        "Tensor? sup, Tensor? sdown, Tensor(a!) sorted, Tensor(b!) tile_expert, Tensor(c!) num_tiles, Tensor(d!) h, "
+        "Tensor(e!) o) -> ()");
   m.def("embed_rows(Tensor ids, Tensor embed, Tensor(a!) resid, Tensor(b!) xb) -> ()");
   m.def("latent_kv_write(Tensor ckr, Tensor norm_w, Tensor positions, Tensor slots, Tensor rope, Tensor(a!) cache, "
         "float eps, Tensor(b!)? vt=None) -> ()");
@@ -402,4 +478,5 @@ TORCH_LIBRARY_IMPL(dsse, CUDA, m) {
   m.impl("lru_scan", &lru_scan);
   m.impl("moe_router", &moe_router);
   m.impl("moe_ffn", &moe_ffn);
+  m.impl("moe_grouped", &moe_grouped);
 }

@@ -8,6 +8,7 @@
 //                fp32 (the residual norm follows).  Each expert's weights are read once per row that chose it: the
 //                decode-shaped path (few rows per expert), and correct for any row count.
 #include "api_layers.h"
+#include "frag.h"
 
 namespace dsse {
 namespace {
@@ -106,6 +107,128 @@ __global__ __launch_bounds__(256) void moe_ffn_kernel(MoeFfnParams p) {
   for (int d = threadIdx.x; d < p.W; d += blockDim.x) p.out[(int64_t)row * p.W + d] = acc[d];
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------------
+// Grouped form: rows sorted by expert, MFMA tiles of 16 rows of ONE expert.  An "id" is a (row, slot) pair,
+// id = row * S + k with S = top (+ 1 when the design has a shared expert: slot `top` is the shared expert, weight 1,
+// expert index E with its own hidden width).  Each expert's weights are read once per 16 of its rows, so the same two
+// GEMM launches serve a decode step (a few rows per expert) and a prompt portion (hundreds).
+//
+//   moe_align     one workgroup: per-expert counts -> tile-padded offsets -> sorted ids (pads -1), the expert of every
+//                 tile and the tile count.  The order of ids inside an expert is whatever the atomics give; a row's
+//                 result does not depend on its place in a tile.
+//   moe_gate_up   h[id, f] = silu(gate_e[f] . x[row]) * (up_e[f] . x[row])       (element type)
+//   moe_down      o[id, :] = weight(id) * down_e . h[id]                          (fp32)
+// The residual norm that follows sums a row's S slots (scalar_norm nsum).
+
+__global__ __launch_bounds__(256) void moe_align_kernel(MoeGroupedParams p) {
+  extern __shared__ int sm[];
+  const int NE = p.E + (p.S > p.top ? 1 : 0);
+  int* cnt = sm;            // [NE]
+  int* off = sm + NE;       // [NE + 1] first sorted position of each expert (multiples of 16)
+  int* fill = off + NE + 1; // [NE]
+  const int n = p.M * p.S;
+  for (int e = threadIdx.x; e < NE; e += blockDim.x) cnt[e] = 0, fill[e] = 0;
+  __syncthreads();
+  for (int id = threadIdx.x; id < n; id += blockDim.x) {
+    const int row = id / p.S, k = id % p.S;
+    int e = k < p.top ? p.topk_idx[row * p.top + k] : p.E;
+    e = (unsigned)e < (unsigned)NE ? e : 0;
+    atomicAdd(&cnt[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0;
+    for (int e = 0; e < NE; ++e) {
+      off[e] = at;
+      at += (cnt[e] + 15) / 16 * 16;
+    }
+    off[NE] = at;
+    *p.num_tiles = at / 16;
+  }
+  __syncthreads();
+  const int total = off[NE];
+  for (int i = threadIdx.x; i < total; i += blockDim.x) p.sorted[i] = -1;
+  for (int e = threadIdx.x; e < NE; e += blockDim.x)
+    for (int t = off[e] / 16; t < off[e + 1] / 16; ++t) p.tile_expert[t] = e;
+  __syncthreads();
+  for (int id = threadIdx.x; id < n; id += blockDim.x) {
+    const int row = id / p.S, k = id % p.S;
+    int e = k < p.top ? p.topk_idx[row * p.top + k] : p.E;
+    e = (unsigned)e < (unsigned)NE ? e : 0;
+    p.sorted[off[e] + atomicAdd(&fill[e], 1)] = id;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gate_up_kernel(MoeGroupedParams p) {
+  using F = Frag<T>;
+  const int t = blockIdx.y;
+  if (t >= *p.num_tiles) return;
+  const int e = p.tile_expert[t];
+  const bool sh = e >= p.E;
+  const int Fe = sh ? p.Fs : p.F;
+  if ((int)blockIdx.x * 64 >= Fe) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
+  const T* gate = sh ? reinterpret_cast<const T*>(p.sgate) : reinterpret_cast<const T*>(p.gate) + (int64_t)e * p.F * p.W;
+  const T* up = sh ? reinterpret_cast<const T*>(p.sup) : reinterpret_cast<const T*>(p.up) + (int64_t)e * p.F * p.W;
+  const int id = p.sorted[t * 16 + r];
+  const bool xv = id >= 0;
+  const T* xr = reinterpret_cast<const T*>(p.x) + (int64_t)(xv ? id / p.S : 0) * p.W;
+  const int f = blockIdx.x * 64 + wave * 16 + r;
+  const bool fv = f < Fe;
+  const T* gr = gate + (int64_t)(fv ? f : 0) * p.W;
+  const T* ur = up + (int64_t)(fv ? f : 0) * p.W;
+  const bool vec = p.vec_w != 0;
+  f32x4 ag = f32x4{0.f, 0.f, 0.f, 0.f}, au = ag;
+  for (int k0 = 0; k0 < p.W; k0 += F::KS) {
+    const int k = k0 + F::PER * g;
+    const typename F::V a = load_frag<T>(xr, k, p.W, xv, vec);
+    ag = mma(a, load_frag<T>(gr, k, p.W, fv, vec), ag);
+    au = mma(a, load_frag<T>(ur, k, p.W, fv, vec), au);
+  }
+  if (!fv) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int id2 = p.sorted[t * 16 + 4 * g + i];
+    if (id2 < 0) continue;
+    const float gv = ag[i];
+    reinterpret_cast<T*>(p.h)[(int64_t)id2 * p.ldh + f] = (T)(gv / (1.0f + expf(-gv)) * au[i]);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_down_kernel(MoeGroupedParams p) {
+  using F = Frag<T>;
+  const int t = blockIdx.y;
+  if (t >= *p.num_tiles) return;
+  const int e = p.tile_expert[t];
+  const bool sh = e >= p.E;
+  const int Fe = sh ? p.Fs : p.F;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
+  const T* down = sh ? reinterpret_cast<const T*>(p.sdown) : reinterpret_cast<const T*>(p.down) + (int64_t)e * p.W * p.F;
+  const int id = p.sorted[t * 16 + r];
+  const bool hv = id >= 0;
+  const T* hr = reinterpret_cast<const T*>(p.h) + (int64_t)(hv ? id : 0) * p.ldh;
+  const int d = blockIdx.x * 64 + wave * 16 + r;
+  const bool dv = d < p.W;
+  const T* dr = down + (int64_t)(dv ? d : 0) * Fe;
+  const bool vech = p.vec_h != 0, vecd = p.vec_h != 0 && Fe % F::PER == 0;
+  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < Fe; k0 += F::KS) {
+    const int k = k0 + F::PER * g;
+    acc = mma(load_frag<T>(hr, k, Fe, hv, vech), load_frag<T>(dr, k, Fe, dv, vecd), acc);
+  }
+  if (!dv) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int id2 = p.sorted[t * 16 + 4 * g + i];
+    if (id2 < 0) continue;
+    const int row = id2 / p.S, k = id2 % p.S;
+    const float wgt = k < p.top ? p.topk_w[row * p.top + k] : 1.0f;
+    p.o[(int64_t)id2 * p.W + d] = wgt * acc[i];
+  }
+}
 }  // namespace
 }  // namespace dsse
 
@@ -124,5 +247,21 @@ extern "C" hipError_t dsse_moe_ffn(const dsse::MoeFfnParams* p, hipStream_t st) 
   if (lds > 64 * 1024) return hipErrorInvalidValue;
   if (p->f32) hipLaunchKernelGGL(dsse::moe_ffn_kernel<float>, dim3(p->M), dim3(256), lds, st, *p);
   else hipLaunchKernelGGL(dsse::moe_ffn_kernel<bf16>, dim3(p->M), dim3(256), lds, st, *p);
+  return hipGetLastError();
+}
+
+extern "C" hipError_t dsse_moe_grouped(const dsse::MoeGroupedParams* p, hipStream_t st) {
+  if (p->M <= 0) return hipSuccess;
+  const int NE = p->E + (p->S > p->top ? 1 : 0);
+  hipLaunchKernelGGL(dsse::moe_align_kernel, dim3(1), dim3(256), sizeof(int) * (3 * NE + 1), st, *p);
+  const int fmax = p->F > p->Fs ? p->F : p->Fs;
+  dim3 g1((fmax + 63) / 64, p->max_tiles), g2((p->W + 63) / 64, p->max_tiles);
+  if (p->f32) {
+    hipLaunchKernelGGL(dsse::moe_gate_up_kernel<float>, g1, dim3(256), 0, st, *p);
+    hipLaunchKernelGGL(dsse::moe_down_kernel<float>, g2, dim3(256), 0, st, *p);
+  } else {
+    hipLaunchKernelGGL(dsse::moe_gate_up_kernel<bf16>, g1, dim3(256), 0, st, *p);
+    hipLaunchKernelGGL(dsse::moe_down_kernel<bf16>, g2, dim3(256), 0, st, *p);
+  }
   return hipGetLastError();
 }

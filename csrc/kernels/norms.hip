@@ -23,18 +23,22 @@ __global__ __launch_bounds__(256) void scalar_norm_kernel(ScalarNormParams p) {
   __shared__ float red[4];
   const int row = blockIdx.x;
   float* resid = p.resid + (int64_t)row * p.W;
-  const float* src = p.mode == 0 ? p.y + (int64_t)row * p.W : resid;
+  const int ns = p.mode == 0 ? p.nsum : 1;
+  const float* src = p.mode == 0 ? p.y + (int64_t)row * ns * p.W : resid;
   T* xb = reinterpret_cast<T*>(p.xb) + (int64_t)row * p.W;
   float ss = 0.f;
   for (int d = threadIdx.x; d < p.W; d += blockDim.x) {
-    const float v = src[d];
+    float v = src[d];
+    for (int s = 1; s < ns; ++s) v += src[(int64_t)s * p.W + d];  // the same order in both passes
     ss += v * v;
   }
   ss = block_sum(ss, red);
   const float s = (float)reinterpret_cast<const T*>(p.g)[0] / sqrtf(ss / (float)p.W + p.eps);
   for (int d = threadIdx.x; d < p.W; d += blockDim.x) {
     if (p.mode == 0) {
-      const float v = resid[d] + src[d] * s;
+      float y = src[d];
+      for (int k = 1; k < ns; ++k) y += src[(int64_t)k * p.W + d];
+      const float v = resid[d] + y * s;
       resid[d] = v;
       xb[d] = (T)v;
     } else {

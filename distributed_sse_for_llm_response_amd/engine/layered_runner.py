@@ -10,7 +10,8 @@ the rows of prompt portions -- that walk the layer list once:
                             -> output GEMM (fp32)
     rglru layer             gelu-branch and input GEMMs (bias / gelu in the epilogue) -> conv_state (slot tail) ->
                             block-diagonal gate GEMM -> lru_scan (slot state) -> output GEMM (fp32)
-    feed-forward            moe_router -> moe_ffn (chosen experts + shared expert, fp32 out)
+    feed-forward            moe_router -> moe_grouped (rows sorted by expert, 16-row MFMA tiles; the shared expert is one
+                            more slot of every row) -> per-slot outputs, summed inside the norm
     after each sublayer     scalar_norm: stream += out / rms(out) * g; xb = rounding
     head                    scalar_norm (final) on the rows that need logits -> GEMM (fp32 logits)
 
@@ -93,6 +94,15 @@ class LayeredRunner(RunnerBase):
             top = max(f.top for f in moe)
             d["tki"] = torch.zeros(M * top, device=dev, dtype=torch.int32)
             d["tkw"] = torch.zeros(M * top, **f32)
+            # grouped experts: ids = (row, slot), slots = top (+ 1: the shared expert)
+            slots = max(f.top + (1 if f.shared_ff else 0) for f in moe)
+            tiles = -(-M * slots // 16) + max(f.experts for f in moe) + 1
+            ldh = -(-max(max(f.ff, f.shared_ff) for f in moe) // 8) * 8
+            d["mo_sorted"] = torch.zeros(tiles * 16, device=dev, dtype=torch.int32)
+            d["mo_tile"] = torch.zeros(tiles, device=dev, dtype=torch.int32)
+            d["mo_n"] = torch.zeros(1, device=dev, dtype=torch.int32)
+            d["mo_h"] = torch.zeros(M * slots, ldh, **el)
+            d["mo_o"] = torch.zeros(M * slots * W, **f32)
         return d
 
     # ------------------------------------------------------------------ layers
@@ -138,11 +148,16 @@ class LayeredRunner(RunnerBase):
                          LRU_DECAY_SCALE)
         ops.gemm_rm(hs, Lw.o, d["y"])
 
-    def _moe(self, f, Fw, M: int, d: dict) -> None:
+    def _moe(self, f, Fw, M: int, d: dict):
+        """Router + grouped experts; returns (per-slot outputs [M * S, W] fp32, S): the norm that follows sums them."""
         tki = d["tki"][:M * f.top].view(M, f.top)
         tkw = d["tkw"][:M * f.top].view(M, f.top)
+        S = f.top + (1 if f.shared_ff else 0)
+        o = d["mo_o"][:M * S * self.cfg.width].view(M * S, self.cfg.width)
         ops.moe_router(d["xb"], Fw.router, Fw.router_b, tki, tkw)
-        ops.moe_ffn(d["xb"], tki, tkw, Fw.gate, Fw.up, Fw.down, Fw.sgate, Fw.sup, Fw.sdown, d["y"])
+        ops.moe_grouped(d["xb"], tki, tkw, Fw.gate, Fw.up, Fw.down, Fw.sgate, Fw.sup, Fw.sdown, d["mo_sorted"],
+                        d["mo_tile"], d["mo_n"], d["mo_h"], o)
+        return o, S
 
     def _layers(self, M: int, d: dict, ids, pos, slots, groups: list, trace: list | None = None) -> None:
         """Embedding + every layer over M packed rows.  `groups`: sequence groups of the step (decode slots, prompt
@@ -157,8 +172,8 @@ class LayeredRunner(RunnerBase):
                 self._recurrent(li, L.mixer, Lw.mix, M, d, groups)
             ops.scalar_norm(d["y"], Lw.norm1, d["resid"], d["xb"], eps)
             if L.mlp is not None:
-                self._moe(L.mlp, Lw.mlp, M, d)
-                ops.scalar_norm(d["y"], Lw.norm2, d["resid"], d["xb"], eps)
+                o, S = self._moe(L.mlp, Lw.mlp, M, d)
+                ops.scalar_norm(o, Lw.norm2, d["resid"], d["xb"], eps, S)
             if trace is not None:
                 trace.append(d["resid"].clone())
 
@@ -180,7 +195,7 @@ class LayeredRunner(RunnerBase):
         r = slice(0, B)
         ops.decode_prep(self.active[r], self.positions[r], self.block_tables[r], self.slots[r], self.ctx_len[r],
                         self.q_len[r], self.kv.num_blocks)
-        d = {k: (v[:B] if v.dim() == 2 else v) for k, v in self._dec.items()}
+        d = {k: (v[:B] if k in ("resid", "xb", "y") else v) for k, v in self._dec.items()}
         self._layers(B, d, self.ids[r], self.positions[r], self.slots[r], [self._decode_group(B)])
         xn = self._dec["xb"][:B]
         ops.scalar_norm(None, self.w.final_norm, d["resid"], xn, self.cfg.eps)

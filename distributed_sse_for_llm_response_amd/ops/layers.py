@@ -29,12 +29,13 @@ def gemm_rm(x, w, out, bias=None, act: int = 0):
         lref.gemm_rm(x, w, out, bias, act)
 
 
-def scalar_norm(y, g, resid, xb, eps: float):
-    """y given: resid += y / rms(y) · g (one number g), xb = resid rounded.  y None: xb = resid / rms(resid) · g."""
+def scalar_norm(y, g, resid, xb, eps: float, nsum: int = 1):
+    """y given: resid += y / rms(y) · g (one number g), xb = resid rounded; y [M · nsum, W] holds each row in nsum
+    consecutive parts that are summed first (the grouped experts' slots).  y None: xb = resid / rms(resid) · g."""
     if _hip(resid):
-        torch.ops.dsse.scalar_norm(y, g, resid, xb, eps)
+        torch.ops.dsse.scalar_norm(y, g, resid, xb, eps, nsum)
     else:
-        lref.scalar_norm(y, g, resid, xb, eps)
+        lref.scalar_norm(y, g, resid, xb, eps, nsum)
 
 
 def embed_rows(ids, embed, resid, xb):
@@ -102,3 +103,14 @@ def moe_ffn(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, out):
         torch.ops.dsse.moe_ffn(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, out)
     else:
         lref.moe_ffn(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, out)
+
+
+def moe_grouped(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, sorted_ids, tile_expert, num_tiles, h, o):
+    """Grouped form of the routed experts: rows sorted by expert, 16-row MFMA tiles of one expert each.  o [M · S, W]
+    (fp32) = weight · expert output per (row, slot), S = top (+ 1: the shared expert's slot); scalar_norm(nsum=S) sums
+    them.  sorted_ids / tile_expert / num_tiles / h are scratch."""
+    if _hip(x):
+        torch.ops.dsse.moe_grouped(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, sorted_ids, tile_expert,
+                                   num_tiles, h, o)
+    else:
+        lref.moe_grouped(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, o)

@@ -27,8 +27,8 @@ def gemm_rm(x, w, out, bias=None, act=0):
     out.copy_(y.to(out.dtype))
 
 
-def scalar_norm(y, g, resid, xb, eps):
-    src = resid if y is None else y
+def scalar_norm(y, g, resid, xb, eps, nsum=1):
+    src = resid if y is None else y.view(resid.shape[0], nsum, -1).sum(1)
     n = src * (g.float().reshape(()) / torch.sqrt(src.pow(2).mean(-1, keepdim=True) + eps))
     if y is None:
         xb.copy_(n.to(xb.dtype))
@@ -169,3 +169,21 @@ def moe_ffn(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, out):
     if sgate is not None:
         acc += ffn(xf, sgate, sup, sdown)
     out.copy_(acc)
+
+
+def moe_grouped(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, o):
+    """o [M * S, W]: slot k < top of row r = weight * expert output, slot `top` = the shared expert."""
+    xf = x.float()
+    M, top = topk_idx.shape
+    S = top + (1 if sgate is not None else 0)
+    ov = o.view(M, S, -1)
+
+    def ffn(h, g, u, d):
+        return (torch.nn.functional.silu(h @ g.float().t()) * (h @ u.float().t())) @ d.float().t()
+
+    for e in range(gate.shape[0]):
+        rows, ks = torch.nonzero(topk_idx == e, as_tuple=True)
+        if rows.numel():
+            ov[rows, ks] = ffn(xf[rows], gate[e], up[e], down[e]) * topk_w[rows, ks].unsqueeze(-1)
+    if sgate is not None:
+        ov[:, top] = ffn(xf, sgate, sup, sdown)

@@ -86,3 +86,37 @@ def test_decode_columns(gpu, H, dn, dr, rk, window):
     rows, flash, ref = _case(gpu, H, dn, dr, rk, window, seqs, 1, seed=7 * H + window)
     assert torch.allclose(rows, ref, atol=3e-2, rtol=3e-2)
     assert torch.allclose(flash, ref, atol=5e-2, rtol=5e-2), float((flash - ref).abs().max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,W,F,Fs,E,top", [(1, 64, 48, 0, 4, 2), (5, 96, 40, 56, 6, 3), (37, 100, 33, 17, 5, 1),
+                                             (300, 128, 96, 64, 12, 4), (64, 72, 24, 24, 3, 3)])
+def test_grouped_experts_against_row_kernel(gpu, dtype, M, W, F, Fs, E, top):
+    """The grouped MFMA form (rows sorted by expert) against the token-major kernel and the PyTorch reference."""
+    g = torch.Generator().manual_seed(M + W)
+    mk = lambda *s: (torch.randn(*s, generator=g) / math.sqrt(s[-1])).to(dtype).to(gpu)  # noqa: E731
+    x = (torch.randn(M, W, generator=g)).to(dtype).to(gpu)
+    router, rb = mk(E, W), (0.1 * torch.randn(E, generator=g)).to(dtype).to(gpu)
+    gate, up, down = mk(E, F, W), mk(E, F, W), mk(E, W, F)
+    sg, su, sd = (mk(Fs, W), mk(Fs, W), mk(W, Fs)) if Fs else (None, None, None)
+    tki = torch.zeros(M, top, dtype=torch.int32, device=gpu)
+    tkw = torch.zeros(M, top, device=gpu)
+    ops.moe_router(x, router, rb, tki, tkw)
+    ri, rw = torch.zeros(M, top, dtype=torch.int32), torch.zeros(M, top)
+    lref.moe_router(x.cpu(), router.cpu(), rb.cpu(), ri, rw)
+    if dtype == torch.float32:
+        assert torch.equal(tki.cpu().sort(-1).values, ri.sort(-1).values)
+    rows = torch.zeros(M, W, device=gpu)
+    ops.moe_ffn(x, tki, tkw, gate, up, down, sg, su, sd, rows)
+    S = top + (1 if Fs else 0)
+    tiles = -(-M * S // 16) + E + 1
+    o = torch.zeros(M * S, W, device=gpu)
+    ops.moe_grouped(x, tki, tkw, gate, up, down, sg, su, sd, torch.zeros(tiles * 16, dtype=torch.int32, device=gpu),
+                    torch.zeros(tiles, dtype=torch.int32, device=gpu), torch.zeros(1, dtype=torch.int32, device=gpu),
+                    torch.zeros(M * S, -(-max(F, Fs) // 8) * 8, dtype=dtype, device=gpu), o)
+    ref = torch.zeros(M * S, W)
+    lref.moe_grouped(x.cpu(), tki.cpu(), tkw.cpu(), gate.cpu(), up.cpu(), down.cpu(), *(t.cpu() if t is not None else None
+                                                                                         for t in (sg, su, sd)), ref)
+    tol = 1e-4 if dtype == torch.float32 else 3e-2
+    assert torch.allclose(o.cpu(), ref, atol=tol, rtol=tol), float((o.cpu() - ref).abs().max())
+    assert torch.allclose(o.view(M, S, W).sum(1).cpu(), rows.cpu(), atol=tol, rtol=tol)
