@@ -34,6 +34,24 @@ sys.path.insert(0, ROOT)
 METRIC = "concurrent SSE streams + p50 inter-token latency, Mistral-7B at 1/2/4/8 MI355X"
 
 
+def family_compare(args):
+    """Prompt-pass and decode-step throughput of several models side by side (same streams, prompt length, steps)."""
+    import torch
+
+    from distributed_sse_for_llm_response_amd.engine import bench_harness
+
+    device = torch.device("cuda", 0) if torch.cuda.is_available() else torch.device("cpu")
+    rows = []
+    for name in args.families.split(","):
+        rows.append(bench_harness.run_family_bench(name.strip(), device=device, streams=args.streams,
+                                                   prompt_len=args.prompt_len, steps=args.steps, warmup=args.warmup))
+        if device.type == "cuda":
+            torch.cuda.empty_cache()
+    print(json.dumps({"metric": "prompt and decode throughput per model family", "unit": "tokens/s", "n_gpus": 1,
+                      "steps": args.steps, "warmup": args.warmup, "dtype": "bf16",
+                      "data": "synthetic prompts, random-init weights", "results": rows}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -48,7 +66,13 @@ def main():
     ap.add_argument("--stub-step-ms", type=float, default=0.0,
                     help="host-path rehearsal only: paced stub replicas emitting one token per stream every "
                          "STUB_STEP_MS instead of the model (router/bus/SSE/client at N GPUs' token rate)")
+    ap.add_argument("--families", default="",
+                    help="comma-separated model names: instead of the headline workload, print prompt and decode "
+                         "throughput of each on its runner (e.g. muderax-mid,mistral-mid); one GPU, --streams, "
+                         "--prompt-len, --steps, --warmup apply")
     args = ap.parse_args()
+    if args.families:
+        return family_compare(args)
 
     from distributed_sse_for_llm_response_amd.engine import bench_harness
 

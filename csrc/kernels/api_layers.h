@@ -65,12 +65,18 @@ struct LatentAttnParams {
   int H, dn, dr, rk, window, qt, rope_len;
   float scale;
   int f32;
+  // MFMA form with the keys of an item split over gridDim.z partitions (decode: few items, long windows): partition z
+  // leaves its unnormalised O^T and (max, sum) per column in part [item][head tile][z][16 x rk | 16 x 2] and a combine
+  // kernel merges them.  nparts <= 1: no split.
+  float* part;
+  int nparts;
 };
 
 struct ConvStateParams {
   const float* in;       // [T, C] fp32
   const void* taps;      // [C, K] (last column = the current token)
   const void* bias;      // [C]
+  const void* in_bias;   // [C] or null: added to every input (the input projection's bias; tails hold biased inputs)
   float* tail;           // [slots, K - 1, C] last K - 1 inputs of each sequence
   const int* q_start;
   const int* q_len;
@@ -78,14 +84,16 @@ struct ConvStateParams {
   const int* state_slot;
   float* out;            // [T, C] fp32
   void* out_b;           // [T, C] element type (the gates' GEMM input)
-  int nseq, C, K;
+  int nseq, C, K, rows;  // rows = T
   int f32;
 };
 
 struct LruScanParams {
   const float* u;        // [T, C] convolution output
-  const float* gates;    // [T, blocks, 2 * bw]: per block [recurrence gate | input gate] pre-activations (bias added)
-  const void* y;         // [T, C] gelu branch
+  const float* gates;    // [T, blocks, 2 * bw]: per block [recurrence gate | input gate] pre-activations (bias added);
+                         // overwritten with the recurrence's coefficients (a | b) when coeff is set
+  const float* y;        // [T, C] gelu branch before its bias and gelu
+  const void* y_bias;    // [C] or null
   const void* lam;       // [C]
   float* state;          // [slots, C]
   const int* q_start;
@@ -93,7 +101,8 @@ struct LruScanParams {
   const int* ctx_len;
   const int* state_slot;
   void* out;             // [T, C] element type: state * y
-  int nseq, C, bw;
+  int nseq, C, bw, rows; // rows = T
+  int coeff;             // 1: compute (a, b) for all rows first; 0: gates already hold them (a later sequence group)
   float c;               // 8: log a = -c r softplus(lam)
   int f32;
 };
@@ -133,7 +142,7 @@ struct MoeGroupedParams {
   const void* sgate;     // shared expert (slot `top`, expert index E) or null
   const void* sup;
   const void* sdown;
-  int* sorted;           // [max_tiles * 16] ids (row * S + slot) grouped by expert, -1 = pad
+  int* sorted;           // [max_tiles * 64] ids (row * S + slot) grouped by expert, -1 = pad
   int* tile_expert;      // [max_tiles]
   int* num_tiles;        // [1]
   void* h;               // [M * S, ldh] element type
@@ -162,4 +171,5 @@ hipError_t dsse_lru_scan(const dsse::LruScanParams* p, hipStream_t st);
 hipError_t dsse_moe_router(const dsse::MoeRouterParams* p, hipStream_t st);
 hipError_t dsse_moe_ffn(const dsse::MoeFfnParams* p, hipStream_t st);
 hipError_t dsse_moe_grouped(const dsse::MoeGroupedParams* p, hipStream_t st);
+hipError_t dsse_moe_topk(const float* z, int M, int E, int top, int* topk_idx, float* topk_w, hipStream_t st);
 }

@@ -168,7 +168,7 @@ void latent_kv_write(const Tensor& ckr, const Tensor& norm_w, const Tensor& posi
 void latent_attention(const Tensor& q, const Tensor& q_abs, const Tensor& cache, const Tensor& block_tables,
                       const Tensor& q_start, const Tensor& q_len, const Tensor& ctx_len, const Tensor& work_seq,
                       const Tensor& work_tile, const Tensor& rope, Tensor& out, int64_t window, double scale,
-                      int64_t qt, const OptTensor& vt, int64_t hp) {
+                      int64_t qt, const OptTensor& vt, int64_t hp, const OptTensor& part, int64_t nparts) {
   gpu(q, "q");
   f32t(q_abs, "q_abs");
   gpu(cache, "cache");
@@ -219,6 +219,14 @@ void latent_attention(const Tensor& q, const Tensor& q_abs, const Tensor& cache,
                 "vt must be [pages, rk, 32]");
     TORCH_CHECK(qt * hp == 16 && (rk == 64 || rk == 128 || rk == 256 || rk == 512) && dr % 32 == 0,
                 "the MFMA form needs qt * hp = 16, rk in {64, 128, 256, 512}, dr % 32 == 0");
+    if (nparts > 1) {
+      TORCH_CHECK(part.has_value(), "a key split needs the part scratch");
+      f32t(*part, "part");
+      const int64_t need = (int64_t)work_seq.numel() * ((H + hp - 1) / hp) * nparts * 16 * (rk + 2);
+      TORCH_CHECK(part->numel() >= need && nparts <= 64, "part scratch too small: ", part->numel(), " < ", need);
+      p.part = part->data_ptr<float>();
+      p.nparts = (int)nparts;
+    }
     DSSE_CHECK_HIP(dsse_latent_flash((int)work_seq.numel(), &p, vt->data_ptr(), (int)qt, (int)hp, cur_stream()));
     return;
   }
@@ -236,7 +244,8 @@ void seq_meta(const Tensor& q_start, const Tensor& q_len, const Tensor& ctx_len,
 }
 
 void conv_state(const Tensor& in, const Tensor& taps, const OptTensor& bias, Tensor& tail, const Tensor& q_start,
-                const Tensor& q_len, const Tensor& ctx_len, const Tensor& state_slot, Tensor& out, Tensor& out_b) {
+                const Tensor& q_len, const Tensor& ctx_len, const Tensor& state_slot, Tensor& out, Tensor& out_b,
+                const OptTensor& in_bias) {
   f32t(in, "in");
   gpu(taps, "taps");
   f32t(tail, "tail");
@@ -264,22 +273,28 @@ void conv_state(const Tensor& in, const Tensor& taps, const OptTensor& bias, Ten
   p.state_slot = state_slot.data_ptr<int>();
   p.out = out.data_ptr<float>();
   p.out_b = out_b.data_ptr();
-  p.C = C, p.K = K;
+  if (in_bias.has_value()) {
+    gpu(*in_bias, "in_bias");
+    same(taps, *in_bias, "in_bias");
+    TORCH_CHECK(in_bias->numel() == C, "in_bias must be [C]");
+    p.in_bias = in_bias->data_ptr();
+  }
+  p.C = C, p.K = K, p.rows = (int)in.size(0);
+  TORCH_CHECK(p.nseq <= 65535 && (p.rows + 31) / 32 <= 65535, "conv_state: grid too large");
   p.f32 = elem(taps, "taps");
   DSSE_CHECK_HIP(dsse_conv_state(&p, cur_stream()));
 }
 
-void lru_scan(const Tensor& u, const Tensor& gates, const Tensor& y, const Tensor& lam, Tensor& state,
+void lru_scan(const Tensor& u, Tensor& gates, const Tensor& y, const Tensor& lam, Tensor& state,
               const Tensor& q_start, const Tensor& q_len, const Tensor& ctx_len, const Tensor& state_slot, Tensor& out,
-              double c) {
+              double c, const OptTensor& y_bias, bool coeff) {
   f32t(u, "u");
   f32t(gates, "gates");
-  gpu(y, "y");
+  f32t(y, "y");
   gpu(lam, "lam");
   f32t(state, "state");
   gpu(out, "out");
-  same(y, lam, "lam");
-  same(y, out, "out");
+  same(lam, out, "out");
   dsse::LruScanParams p{};
   seq_meta(q_start, q_len, ctx_len, state_slot, p.nseq);
   const int C = (int)u.size(1);
@@ -289,7 +304,15 @@ void lru_scan(const Tensor& u, const Tensor& gates, const Tensor& y, const Tenso
   TORCH_CHECK(state.dim() == 2 && state.size(1) == C, "state must be [slots, C]");
   p.u = u.data_ptr<float>();
   p.gates = gates.data_ptr<float>();
-  p.y = y.data_ptr();
+  p.y = y.data_ptr<float>();
+  if (y_bias.has_value()) {
+    gpu(*y_bias, "y_bias");
+    same(lam, *y_bias, "y_bias");
+    TORCH_CHECK(y_bias->numel() == C, "y_bias must be [C]");
+    p.y_bias = y_bias->data_ptr();
+  }
+  p.rows = (int)u.size(0);
+  p.coeff = coeff ? 1 : 0;
   p.lam = lam.data_ptr();
   p.state = state.data_ptr<float>();
   p.q_start = q_start.data_ptr<int>();
@@ -299,7 +322,7 @@ void lru_scan(const Tensor& u, const Tensor& gates, const Tensor& y, const Tenso
   p.out = out.data_ptr();
   p.C = C, p.bw = (int)gates.size(2) / 2;
   p.c = (float)c;
-  p.f32 = elem(y, "y");
+  p.f32 = elem(lam, "lam");
   DSSE_CHECK_HIP(dsse_lru_scan(&p, cur_stream()));
 }
 
@@ -375,8 +398,8 @@ void moe_ffn(const Tensor& x, const Tensor& topk_idx, const Tensor& topk_w, cons
 }
 
 // Grouped form of the routed experts: o [M * S, W] (fp32) = per-(row, slot) expert outputs times their weights, S = top
-// (+ 1 with a shared expert); the caller sums a row's S parts (scalar_norm nsum).  Scratch: sorted [tiles * 16],
-// tile_expert [tiles], num_tiles [1] (int32), h [M * S, ldh] (element type), tiles >= ceil(M S / 16) + experts.
+// (+ 1 with a shared expert); the caller sums a row's S parts (scalar_norm nsum).  Scratch: sorted [tiles * 64],
+// tile_expert [tiles], num_tiles [1] (int32), h [M * S, ldh] (element type), tiles >= ceil(M S / 64) + experts + 1.
 void moe_grouped(const Tensor& x, const Tensor& topk_idx, const Tensor& topk_w, const Tensor& gate, const Tensor& up,
                  const Tensor& down, const OptTensor& sgate, const OptTensor& sup, const OptTensor& sdown, Tensor& sorted,
                  Tensor& tile_expert, Tensor& num_tiles, Tensor& h, Tensor& o) {
@@ -421,7 +444,7 @@ void moe_grouped(const Tensor& x, const Tensor& topk_idx, const Tensor& topk_w, 
   }
   const int64_t ids = (int64_t)p.M * p.S;
   p.max_tiles = (int)tile_expert.numel();
-  TORCH_CHECK(p.max_tiles >= (ids + 15) / 16 + p.E + 1 && sorted.numel() >= (int64_t)p.max_tiles * 16 && p.max_tiles <= 65535,
+  TORCH_CHECK(p.max_tiles >= (ids + 63) / 64 + p.E + 1 && sorted.numel() >= (int64_t)p.max_tiles * 64 && p.max_tiles <= 65535,
               "moe_grouped: scratch too small for ", ids, " ids");
   TORCH_CHECK(h.dim() == 2 && h.size(0) >= ids && h.size(1) >= std::max(p.F, p.Fs) && o.dim() == 2 && o.size(0) == ids &&
                   o.size(1) == p.W && p.E + 1 <= 4096,
@@ -445,6 +468,18 @@ void moe_grouped(const Tensor& x, const Tensor& topk_idx, const Tensor& topk_w, 
   DSSE_CHECK_HIP(dsse_moe_grouped(&p, cur_stream()));
 }
 
+void moe_topk(const Tensor& logits, Tensor& topk_idx, Tensor& topk_w) {
+  f32t(logits, "logits");
+  i32(topk_idx, "topk_idx");
+  f32t(topk_w, "topk_w");
+  const int M = (int)logits.size(0), E = (int)logits.size(1), top = (int)topk_idx.size(1);
+  TORCH_CHECK(logits.dim() == 2 && topk_idx.dim() == 2 && topk_idx.size(0) == M && topk_w.sizes() == topk_idx.sizes() &&
+                  top >= 1 && top <= E,
+              "moe_topk shapes");
+  DSSE_CHECK_HIP(dsse_moe_topk(logits.data_ptr<float>(), M, E, top, topk_idx.data_ptr<int>(), topk_w.data_ptr<float>(),
+                               cur_stream()));
+}
+
 }  // namespace
 
 TORCH_LIBRARY_FRAGMENT(dsse, m) {
@@ -458,12 +493,13 @@ TORCH_LIBRARY_FRAGMENT(dsse, m) {
         "float eps, Tensor(b!)? vt=None) -> ()");
   m.def("latent_attention(Tensor q, Tensor q_abs, Tensor cache, Tensor block_tables, Tensor q_start, Tensor q_len, "
         "Tensor ctx_len, Tensor work_seq, Tensor work_tile, Tensor rope, Tensor(a!) out, int window, float scale, "
-        "int qt, Tensor? vt=None, int hp=1) -> ()");
+        "int qt, Tensor? vt=None, int hp=1, Tensor(b!)? part=None, int nparts=1) -> ()");
   m.def("conv_state(Tensor inp, Tensor taps, Tensor? bias, Tensor(a!) tail, Tensor q_start, Tensor q_len, "
-        "Tensor ctx_len, Tensor state_slot, Tensor(b!) out, Tensor(c!) out_b) -> ()");
-  m.def("lru_scan(Tensor u, Tensor gates, Tensor y, Tensor lam, Tensor(a!) state, Tensor q_start, Tensor q_len, "
-        "Tensor ctx_len, Tensor state_slot, Tensor(b!) out, float c) -> ()");
+        "Tensor ctx_len, Tensor state_slot, Tensor(b!) out, Tensor(c!) out_b, Tensor? in_bias=None) -> ()");
+  m.def("lru_scan(Tensor u, Tensor(c!) gates, Tensor y, Tensor lam, Tensor(a!) state, Tensor q_start, Tensor q_len, "
+        "Tensor ctx_len, Tensor state_slot, Tensor(b!) out, float c, Tensor? y_bias=None, bool coeff=True) -> ()");
   m.def("moe_router(Tensor x, Tensor w, Tensor? b, Tensor(a!) topk_idx, Tensor(b!) topk_w) -> ()");
+  m.def("moe_topk(Tensor logits, Tensor(a!) topk_idx, Tensor(b!) topk_w) -> ()");
   m.def("moe_ffn(Tensor x, Tensor topk_idx, Tensor topk_w, Tensor gate, Tensor up, Tensor down, Tensor? sgate, "
         "Tensor? sup, Tensor? sdown, Tensor(a!) out) -> ()");
 }
@@ -477,6 +513,7 @@ TORCH_LIBRARY_IMPL(dsse, CUDA, m) {
   m.impl("conv_state", &conv_state);
   m.impl("lru_scan", &lru_scan);
   m.impl("moe_router", &moe_router);
+  m.impl("moe_topk", &moe_topk);
   m.impl("moe_ffn", &moe_ffn);
   m.impl("moe_grouped", &moe_grouped);
 }

@@ -217,7 +217,14 @@ __global__ __launch_bounds__(64) void latent_flash_kernel(LatentAttnParams p, co
   for (int n = 0; n < NT; ++n) O[n] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
   const int nks = D / 32;
-  for (int pg = lo / kBS; pg <= hi / kBS; ++pg) {
+  int pg0 = lo / kBS, pg1 = hi / kBS;
+  const int np = p.nparts > 1 ? p.nparts : 1;
+  if (np > 1) {  // this partition's share of the pages (even split of the item's own range)
+    const int per = (pg1 - pg0 + np) / np;
+    pg0 += blockIdx.z * per;
+    pg1 = pg0 + per - 1 < pg1 ? pg0 + per - 1 : pg1;
+  }
+  for (int pg = pg0; pg <= pg1; ++pg) {
     int blk = bt[pg];
     blk = (unsigned)blk < (unsigned)p.num_blocks ? blk : 0;
     const bf16* krow0 = rows + ((int64_t)blk * kBS + r) * D + 8 * g;        // key r of the page's first half
@@ -260,6 +267,18 @@ __global__ __launch_bounds__(64) void latent_flash_kernel(LatentAttnParams p, co
       O[n] = mfma16x16x32(ld_bf16x8(vrow + (int64_t)n * 16 * kBS), pf, o);
     }
   }
+  if (np > 1) {
+    float* po = p.part + (((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * np + blockIdx.z) * (16 * (p.rk + 2));
+#pragma unroll
+    for (int n = 0; n < NT; ++n)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) po[r * p.rk + 16 * n + 4 * g + i] = O[n][i];
+    if (g == 0) {
+      po[16 * p.rk + 2 * r] = m;
+      po[16 * p.rk + 2 * r + 1] = l;
+    }
+    return;
+  }
   if (c_ok) {
     bf16* out = reinterpret_cast<bf16*>(p.out) + (c_row * p.H + c_head) * p.rk;
     const float inv = l > 0.f ? 1.0f / l : 0.0f;
@@ -270,6 +289,34 @@ __global__ __launch_bounds__(64) void latent_flash_kernel(LatentAttnParams p, co
       for (int i = 0; i < 4; ++i) v[i] = (bf16)(O[n][i] * inv);
       *reinterpret_cast<bf16x4*>(out + 16 * n + 4 * g) = v;
     }
+  }
+}
+
+// Merge of the key partitions of latent_flash_kernel: per column, M = max of the partitions' maxima,
+// out = sum_z e^(m_z - M) O_z / sum_z e^(m_z - M) l_z.
+__global__ __launch_bounds__(256) void latent_flash_combine_kernel(LatentAttnParams p, int rt, int hp) {
+  const int seq = p.work_seq[blockIdx.x], tile = p.work_tile[blockIdx.x];
+  const int ql = p.q_len[seq];
+  if (tile * rt >= ql) return;
+  const int np = p.nparts;
+  const int stride = 16 * (p.rk + 2);
+  const float* base = p.part + ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * np * stride;
+  for (int idx = threadIdx.x; idx < 16 * p.rk; idx += blockDim.x) {
+    const int col = idx / p.rk, d = idx % p.rk;
+    const int off = tile * rt + col / hp, head = blockIdx.y * hp + col % hp;
+    if (off >= ql || head >= p.H) continue;
+    float M = -INFINITY;
+    for (int z = 0; z < np; ++z) M = fmaxf(M, base[z * stride + 16 * p.rk + 2 * col]);
+    float num = 0.f, den = 0.f;
+    for (int z = 0; z < np; ++z) {
+      const float mz = base[z * stride + 16 * p.rk + 2 * col];
+      if (mz == -INFINITY) continue;
+      const float w = expf(mz - M);
+      num += w * base[z * stride + col * p.rk + d];
+      den += w * base[z * stride + 16 * p.rk + 2 * col + 1];
+    }
+    reinterpret_cast<bf16*>(p.out)[((int64_t)(p.q_start[seq] + off) * p.H + head) * p.rk + d] =
+        (bf16)(den > 0.f ? num / den : 0.0f);
   }
 }
 
@@ -319,7 +366,9 @@ extern "C" hipError_t dsse_latent_flash(int num_work, const dsse::LatentAttnPara
   if (num_work <= 0) return hipSuccess;
   if (p->f32 || rt * hp != 16 || p->rk % 32 || p->dr % 32) return hipErrorInvalidValue;
   const size_t lds = 16 * (size_t)(p->rk + p->dr + 8) * sizeof(bf16);
-  dim3 grid(num_work, (p->H + hp - 1) / hp);
+  const int np = p->nparts > 1 ? p->nparts : 1;
+  if (np > 1 && !p->part) return hipErrorInvalidValue;
+  dim3 grid(num_work, (p->H + hp - 1) / hp, np);
   const bf16* v = reinterpret_cast<const bf16*>(vt);
   switch (p->rk / 16) {
     case 4: hipLaunchKernelGGL(dsse::latent_flash_kernel<4>, grid, dim3(64), lds, st, *p, v, rt, hp); break;
@@ -328,5 +377,7 @@ extern "C" hipError_t dsse_latent_flash(int num_work, const dsse::LatentAttnPara
     case 32: hipLaunchKernelGGL(dsse::latent_flash_kernel<32>, grid, dim3(64), lds, st, *p, v, rt, hp); break;
     default: return hipErrorInvalidValue;
   }
+  if (np > 1)
+    hipLaunchKernelGGL(dsse::latent_flash_combine_kernel, dim3(num_work, (p->H + hp - 1) / hp), dim3(256), 0, st, *p, rt, hp);
   return hipGetLastError();
 }

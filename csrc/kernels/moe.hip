@@ -52,6 +52,37 @@ __global__ __launch_bounds__(64) void moe_router_kernel(MoeRouterParams p) {
   }
 }
 
+// The choice alone, from fp32 logits [M, E] (the router's GEMM, bias added): one thread per row.
+__global__ __launch_bounds__(256) void moe_topk_kernel(const float* __restrict__ z, int M, int E, int top, int* topk_idx,
+                                                       float* topk_w) {
+  const int row = blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= M) return;
+  const float* zr = z + (int64_t)row * E;
+  int* idx = topk_idx + (int64_t)row * top;
+  float* wt = topk_w + (int64_t)row * top;
+  float mx = 0.f;
+  for (int k = 0; k < top; ++k) {
+    int best = -1;
+    float bv = 0.f;
+    for (int e = 0; e < E; ++e) {
+      bool used = false;
+      for (int j = 0; j < k; ++j) used |= idx[j] == e;
+      if (used) continue;
+      const float v = zr[e];
+      if (best < 0 || v > bv) best = e, bv = v;
+    }
+    idx[k] = best < 0 ? 0 : best;
+    wt[k] = bv;
+    if (k == 0) mx = bv;
+  }
+  float sum = 0.f;
+  for (int k = 0; k < top; ++k) {
+    wt[k] = expf(wt[k] - mx);
+    sum += wt[k];
+  }
+  for (int k = 0; k < top; ++k) wt[k] /= sum;
+}
+
 template <typename T>
 DEV void expert_row(const T* gate, const T* up, const T* down, int W, int F, float wgt, const float* xs, float* hs,
                     float* acc) {
@@ -111,7 +142,7 @@ __global__ __launch_bounds__(256) void moe_ffn_kernel(MoeFfnParams p) {
 // ---------------------------------------------------------------------------------------------------------------------
 // Grouped form: rows sorted by expert, MFMA tiles of 16 rows of ONE expert.  An "id" is a (row, slot) pair,
 // id = row * S + k with S = top (+ 1 when the design has a shared expert: slot `top` is the shared expert, weight 1,
-// expert index E with its own hidden width).  Each expert's weights are read once per 16 of its rows, so the same two
+// expert index E with its own hidden width).  Each expert's weights are read once per 64 of its rows (four 16-row MFMA tiles; empty ones are skipped), so the same two
 // GEMM launches serve a decode step (a few rows per expert) and a prompt portion (hundreds).
 //
 //   moe_align     one workgroup: per-expert counts -> tile-padded offsets -> sorted ids (pads -1), the expert of every
@@ -121,11 +152,13 @@ __global__ __launch_bounds__(256) void moe_ffn_kernel(MoeFfnParams p) {
 //   moe_down      o[id, :] = weight(id) * down_e . h[id]                          (fp32)
 // The residual norm that follows sums a row's S slots (scalar_norm nsum).
 
+constexpr int kMoeRows = 64;  // rows of one expert per workgroup tile: four 16-row MFMA tiles share every weight fragment
+
 __global__ __launch_bounds__(256) void moe_align_kernel(MoeGroupedParams p) {
   extern __shared__ int sm[];
   const int NE = p.E + (p.S > p.top ? 1 : 0);
   int* cnt = sm;            // [NE]
-  int* off = sm + NE;       // [NE + 1] first sorted position of each expert (multiples of 16)
+  int* off = sm + NE;       // [NE + 1] first sorted position of each expert (multiples of kMoeRows)
   int* fill = off + NE + 1; // [NE]
   const int n = p.M * p.S;
   for (int e = threadIdx.x; e < NE; e += blockDim.x) cnt[e] = 0, fill[e] = 0;
@@ -141,16 +174,16 @@ __global__ __launch_bounds__(256) void moe_align_kernel(MoeGroupedParams p) {
     int at = 0;
     for (int e = 0; e < NE; ++e) {
       off[e] = at;
-      at += (cnt[e] + 15) / 16 * 16;
+      at += (cnt[e] + kMoeRows - 1) / kMoeRows * kMoeRows;
     }
     off[NE] = at;
-    *p.num_tiles = at / 16;
+    *p.num_tiles = at / kMoeRows;
   }
   __syncthreads();
   const int total = off[NE];
   for (int i = threadIdx.x; i < total; i += blockDim.x) p.sorted[i] = -1;
   for (int e = threadIdx.x; e < NE; e += blockDim.x)
-    for (int t = off[e] / 16; t < off[e + 1] / 16; ++t) p.tile_expert[t] = e;
+    for (int t = off[e] / kMoeRows; t < off[e + 1] / kMoeRows; ++t) p.tile_expert[t] = e;
   __syncthreads();
   for (int id = threadIdx.x; id < n; id += blockDim.x) {
     const int row = id / p.S, k = id % p.S;
@@ -172,28 +205,47 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(MoeGroupedParams p) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
   const T* gate = sh ? reinterpret_cast<const T*>(p.sgate) : reinterpret_cast<const T*>(p.gate) + (int64_t)e * p.F * p.W;
   const T* up = sh ? reinterpret_cast<const T*>(p.sup) : reinterpret_cast<const T*>(p.up) + (int64_t)e * p.F * p.W;
-  const int id = p.sorted[t * 16 + r];
-  const bool xv = id >= 0;
-  const T* xr = reinterpret_cast<const T*>(p.x) + (int64_t)(xv ? id / p.S : 0) * p.W;
+  const int* ids = p.sorted + t * kMoeRows;
+  // an expert's ids fill its tiles from the front: a 16-row sub-tile is empty when its first id is a pad
+  const T* xr[4];
+  bool xv[4], live[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int id = ids[16 * i + r];
+    live[i] = ids[16 * i] >= 0;
+    xv[i] = id >= 0;
+    xr[i] = reinterpret_cast<const T*>(p.x) + (int64_t)(xv[i] ? id / p.S : 0) * p.W;
+  }
   const int f = blockIdx.x * 64 + wave * 16 + r;
   const bool fv = f < Fe;
   const T* gr = gate + (int64_t)(fv ? f : 0) * p.W;
   const T* ur = up + (int64_t)(fv ? f : 0) * p.W;
   const bool vec = p.vec_w != 0;
-  f32x4 ag = f32x4{0.f, 0.f, 0.f, 0.f}, au = ag;
+  f32x4 ag[4], au[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) ag[i] = au[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int k0 = 0; k0 < p.W; k0 += F::KS) {
     const int k = k0 + F::PER * g;
-    const typename F::V a = load_frag<T>(xr, k, p.W, xv, vec);
-    ag = mma(a, load_frag<T>(gr, k, p.W, fv, vec), ag);
-    au = mma(a, load_frag<T>(ur, k, p.W, fv, vec), au);
+    const typename F::V bg = load_frag<T>(gr, k, p.W, fv, vec), bu = load_frag<T>(ur, k, p.W, fv, vec);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (!live[i]) continue;  // uniform over the workgroup
+      const typename F::V a = load_frag<T>(xr[i], k, p.W, xv[i], vec);
+      ag[i] = mma(a, bg, ag[i]);
+      au[i] = mma(a, bu, au[i]);
+    }
   }
   if (!fv) return;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int id2 = p.sorted[t * 16 + 4 * g + i];
-    if (id2 < 0) continue;
-    const float gv = ag[i];
-    reinterpret_cast<T*>(p.h)[(int64_t)id2 * p.ldh + f] = (T)(gv / (1.0f + expf(-gv)) * au[i]);
+    if (!live[i]) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int id2 = ids[16 * i + 4 * g + j];
+      if (id2 < 0) continue;
+      const float gv = ag[i][j];
+      reinterpret_cast<T*>(p.h)[(int64_t)id2 * p.ldh + f] = (T)(gv / (1.0f + expf(-gv)) * au[i][j]);
+    }
   }
 }
 
@@ -207,28 +259,47 @@ __global__ __launch_bounds__(256) void moe_down_kernel(MoeGroupedParams p) {
   const int Fe = sh ? p.Fs : p.F;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
   const T* down = sh ? reinterpret_cast<const T*>(p.sdown) : reinterpret_cast<const T*>(p.down) + (int64_t)e * p.W * p.F;
-  const int id = p.sorted[t * 16 + r];
-  const bool hv = id >= 0;
-  const T* hr = reinterpret_cast<const T*>(p.h) + (int64_t)(hv ? id : 0) * p.ldh;
+  const int* ids = p.sorted + t * kMoeRows;
+  const T* hr[4];
+  bool hv[4], live[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int id = ids[16 * i + r];
+    live[i] = ids[16 * i] >= 0;
+    hv[i] = id >= 0;
+    hr[i] = reinterpret_cast<const T*>(p.h) + (int64_t)(hv[i] ? id : 0) * p.ldh;
+  }
   const int d = blockIdx.x * 64 + wave * 16 + r;
   const bool dv = d < p.W;
   const T* dr = down + (int64_t)(dv ? d : 0) * Fe;
   const bool vech = p.vec_h != 0, vecd = p.vec_h != 0 && Fe % F::PER == 0;
-  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+  f32x4 acc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int k0 = 0; k0 < Fe; k0 += F::KS) {
     const int k = k0 + F::PER * g;
-    acc = mma(load_frag<T>(hr, k, Fe, hv, vech), load_frag<T>(dr, k, Fe, dv, vecd), acc);
+    const typename F::V b = load_frag<T>(dr, k, Fe, dv, vecd);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (!live[i]) continue;
+      acc[i] = mma(load_frag<T>(hr[i], k, Fe, hv[i], vech), b, acc[i]);
+    }
   }
   if (!dv) return;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int id2 = p.sorted[t * 16 + 4 * g + i];
-    if (id2 < 0) continue;
-    const int row = id2 / p.S, k = id2 % p.S;
-    const float wgt = k < p.top ? p.topk_w[row * p.top + k] : 1.0f;
-    p.o[(int64_t)id2 * p.W + d] = wgt * acc[i];
+    if (!live[i]) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int id2 = ids[16 * i + 4 * g + j];
+      if (id2 < 0) continue;
+      const int row = id2 / p.S, k = id2 % p.S;
+      const float wgt = k < p.top ? p.topk_w[row * p.top + k] : 1.0f;
+      p.o[(int64_t)id2 * p.W + d] = wgt * acc[i][j];
+    }
   }
 }
+
 }  // namespace
 }  // namespace dsse
 
@@ -263,5 +334,11 @@ extern "C" hipError_t dsse_moe_grouped(const dsse::MoeGroupedParams* p, hipStrea
     hipLaunchKernelGGL(dsse::moe_gate_up_kernel<bf16>, g1, dim3(256), 0, st, *p);
     hipLaunchKernelGGL(dsse::moe_down_kernel<bf16>, g2, dim3(256), 0, st, *p);
   }
+  return hipGetLastError();
+}
+
+extern "C" hipError_t dsse_moe_topk(const float* z, int M, int E, int top, int* topk_idx, float* topk_w, hipStream_t st) {
+  if (M <= 0) return hipSuccess;
+  hipLaunchKernelGGL(dsse::moe_topk_kernel, dim3((M + 255) / 256), dim3(256), 0, st, z, M, E, top, topk_idx, topk_w);
   return hipGetLastError();
 }

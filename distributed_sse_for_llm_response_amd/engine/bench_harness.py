@@ -418,3 +418,50 @@ def _sync(device, world):
         import torch.distributed as dist
 
         dist.barrier()
+
+
+def run_family_bench(model: str, device=None, streams: int = 16, prompt_len: int = 1024, steps: int = 32, warmup: int = 4,
+                     seed: int = 0) -> dict:
+    """Prompt and decode throughput of one model (any family of the registry), on the runner alone: every stream's
+    prompt is prefilled whole (the passes after the first are timed: tokens/s of a `prompt_len`-token pass), then
+    `steps` decode steps of all streams at that context are timed (the captured graph on a GPU; tokens/s = streams /
+    step).  Random weights, random prompt tokens."""
+    from ..models import registry
+
+    device = device or torch.device("cuda" if torch.cuda.is_available() else "cpu")
+    cuda = device.type == "cuda"
+    fam, cfg, ckpt = registry.resolve(model)
+    w = registry.load_weights(fam, cfg, ckpt, device=device, seed=1234)
+    max_len = prompt_len + steps + warmup + 2 * PAGE
+    per = blocks_needed(max_len)
+    r = registry.make_runner(fam, w, num_blocks=streams * per + 4, max_batch=streams, max_model_len=max_len,
+                             max_prefill_tokens=max(prompt_len, 64), device=device, use_graphs=cuda)
+    gen = torch.Generator().manual_seed(seed)
+    sync = (lambda: torch.cuda.synchronize(device)) if cuda else (lambda: None)
+    times = []
+    for s in range(streams):
+        blocks = list(range(s * per, (s + 1) * per))
+        r.block_tables[s, :per] = torch.tensor(blocks, dtype=torch.int32)
+        toks = torch.randint(3, cfg.vocab_size, (prompt_len,), generator=gen).tolist()
+        sync()
+        t0 = time.perf_counter()
+        r.prefill([PrefillSeq(s, toks, 0, blocks, True)], ring_row=0)
+        sync()
+        times.append(time.perf_counter() - t0)
+    pf = sorted(times[1:] or times)
+    pf_s = pf[len(pf) // 2]
+    r.active[:streams] = 1
+    r.temperature[:streams] = 1.0
+    if cuda:
+        r.capture([streams])
+    for _ in range(warmup):
+        r.decode(streams)
+    sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        r.decode(streams)
+    sync()
+    step_s = (time.perf_counter() - t0) / steps
+    return {"model": cfg.name, "family": fam.name, "params_resident_gb": round(w.nbytes() / 1e9, 2), "streams": streams,
+            "prompt_len": prompt_len, "prefill_ms": round(pf_s * 1e3, 3), "prefill_tok_s": round(prompt_len / pf_s, 1),
+            "decode_step_ms": round(step_s * 1e3, 4), "decode_tok_s": round(streams / step_s, 1)}

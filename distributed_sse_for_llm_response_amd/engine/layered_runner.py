@@ -8,9 +8,10 @@ the rows of prompt portions -- that walk the layer list once:
                             fold of the unrotated query through the key up-projection -> latent_attention over the
                             window (decode slots: one-row items; portions: tiled items) -> per-head value up-projection
                             -> output GEMM (fp32)
-    rglru layer             gelu-branch and input GEMMs (bias / gelu in the epilogue) -> conv_state (slot tail) ->
-                            block-diagonal gate GEMM -> lru_scan (slot state) -> output GEMM (fp32)
-    feed-forward            moe_router -> moe_grouped (rows sorted by expert, 16-row MFMA tiles; the shared expert is one
+    rglru layer             gelu-branch and input GEMMs (fp32 out) -> conv_state (+ input bias; slot tail) -> block-
+                            diagonal gate GEMM -> lru_scan (coefficients for all rows at once, then the walk over each
+                            sequence's rows with the branch's bias + gelu; slot state) -> output GEMM (fp32)
+    feed-forward            router GEMM (fp32 logits) -> moe_topk -> moe_grouped (rows sorted by expert, 16-row MFMA tiles; the shared expert is one
                             more slot of every row) -> per-slot outputs, summed inside the norm
     after each sublayer     scalar_norm: stream += out / rms(out) * g; xb = rounding
     head                    scalar_norm (final) on the rows that need logits -> GEMM (fp32 logits)
@@ -36,6 +37,7 @@ from .model_runner import RunnerBase, _capture, batch_buckets
 from .weights import LayeredWeights
 
 ATTN_ROWS_TILE = 4    # query rows per work item of the row-wise attention kernel (prompt portions)
+FLASH_DECODE_WAVES = 512  # waves a decode attention launch aims for (two per CU)
 FLASH_ROWS_TILE = 16  # query rows per work item of the MFMA attention form (x 16 / rows heads = 16 columns)
 
 
@@ -68,6 +70,9 @@ class LayeredRunner(RunnerBase):
             if key not in self._rope:
                 self._rope[key] = m.rot.table(max_model_len + 1, m.rot_dim, dev)
         self._dec = self._buffers(max_batch)  # static decode activations (captured graphs read and write them)
+        words = max((ops.latent_flash_part_floats(max_batch, m.heads, 16, 16, m.kv_rank) for i, m in att.items()
+                     if i in flash), default=0)
+        self._flash_part = torch.zeros(max(1, words), device=dev, dtype=torch.float32)
 
     # ------------------------------------------------------------------ buffers
     def _buffers(self, M: int) -> dict:
@@ -87,8 +92,8 @@ class LayeredRunner(RunnerBase):
             d["attn"] = torch.zeros(M * max(m.heads * m.vdim for m in att), **el)
         if rec:
             C = max(m.width for m in rec)
-            d["yb"], d["ub"], d["hs"] = (torch.zeros(M * C, **el) for _ in range(3))
-            d["ux"], d["u"] = (torch.zeros(M * C, **f32) for _ in range(2))
+            d["ub"], d["hs"] = (torch.zeros(M * C, **el) for _ in range(2))
+            d["yr"], d["ux"], d["u"] = (torch.zeros(M * C, **f32) for _ in range(3))
             d["gates"] = torch.zeros(M * 2 * C, **f32)
         if moe:
             top = max(f.top for f in moe)
@@ -96,9 +101,10 @@ class LayeredRunner(RunnerBase):
             d["tkw"] = torch.zeros(M * top, **f32)
             # grouped experts: ids = (row, slot), slots = top (+ 1: the shared expert)
             slots = max(f.top + (1 if f.shared_ff else 0) for f in moe)
-            tiles = -(-M * slots // 16) + max(f.experts for f in moe) + 1
+            tiles = -(-M * slots // 64) + max(f.experts for f in moe) + 2
+            d["mo_z"] = torch.zeros(M * max(f.experts for f in moe), **f32)
             ldh = -(-max(max(f.ff, f.shared_ff) for f in moe) // 8) * 8
-            d["mo_sorted"] = torch.zeros(tiles * 16, device=dev, dtype=torch.int32)
+            d["mo_sorted"] = torch.zeros(tiles * 64, device=dev, dtype=torch.int32)
             d["mo_tile"] = torch.zeros(tiles, device=dev, dtype=torch.int32)
             d["mo_n"] = torch.zeros(1, device=dev, dtype=torch.int32)
             d["mo_h"] = torch.zeros(M * slots, ldh, **el)
@@ -123,29 +129,44 @@ class LayeredRunner(RunnerBase):
         for g in groups:
             if vt is not None:  # MFMA form: a decode row's heads side by side, a portion's rows in tiles of 16
                 dec = g["qt"] == 1
-                ops.latent_attention(q, qabs, cache, g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"] if dec else g["fs"],
-                                     g["wt"] if dec else g["ft"], rope, lat, m.window, m.scale,
-                                     1 if dec else FLASH_ROWS_TILE, vt, 16 if dec else 16 // FLASH_ROWS_TILE)
+                if dec:  # few items: their keys are split over partitions so that the chip is filled
+                    B = g["ws"].numel()
+                    np_ = self._decode_parts(B, H, m.window)
+                    ops.latent_attention(q, qabs, cache, g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"], g["wt"], rope,
+                                         lat, m.window, m.scale, 1, vt, 16, self._flash_part if np_ > 1 else None, np_)
+                else:
+                    ops.latent_attention(q, qabs, cache, g["bt"], g["qs"], g["ql"], g["ctx"], g["fs"], g["ft"], rope,
+                                         lat, m.window, m.scale, FLASH_ROWS_TILE, vt, 16 // FLASH_ROWS_TILE)
             else:
                 ops.latent_attention(q, qabs, cache, g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"], g["wt"], rope, lat,
                                      m.window, m.scale, g["qt"])
         ops.gemm_rm(lat.permute(1, 0, 2), Lw.uv, attn.permute(1, 0, 2))
         ops.gemm_rm(attn.view(M, H * dv), Lw.o, d["y"])
 
+    def _decode_parts(self, B: int, heads: int, window: int) -> int:
+        """Key partitions of the decode attention: enough (item, head tile, partition) waves for the chip, at most one
+        per page that a sequence can hold inside the window, at most 16."""
+        pages = -(-min(window, self.max_model_len) // PAGE) + 1
+        want = -(-FLASH_DECODE_WAVES // max(1, B * (-(-heads // 16))))
+        return max(1, min(16, pages, want))
+
     def _recurrent(self, li: int, m, Lw, M: int, d: dict, groups: list) -> None:
         C, nb = m.width, m.blocks
         bw = C // nb
-        yb, ub, hs = (d[k][:M * C].view(M, C) for k in ("yb", "ub", "hs"))
-        ux, u = (d[k][:M * C].view(M, C) for k in ("ux", "u"))
+        ub, hs = (d[k][:M * C].view(M, C) for k in ("ub", "hs"))
+        yr, ux, u = (d[k][:M * C].view(M, C) for k in ("yr", "ux", "u"))
         gates = d["gates"][:M * 2 * C].view(M, nb, 2 * bw)
-        ops.gemm_rm(d["xb"], Lw.y, yb, bias=Lw.y_b, act=1)
-        ops.gemm_rm(d["xb"], Lw.x, ux, bias=Lw.x_b)
+        # both input projections leave fp32 without bias: the convolution adds its input's bias, the scan applies
+        # the branch's bias and gelu
+        ops.gemm_rm(d["xb"], Lw.y, yr)
+        ops.gemm_rm(d["xb"], Lw.x, ux)
         for g in groups:
-            ops.conv_state(ux, Lw.conv, Lw.conv_b, self.state.tail[li], g["qs"], g["ql"], g["ctx"], g["ss"], u, ub)
+            ops.conv_state(ux, Lw.conv, Lw.conv_b, self.state.tail[li], g["qs"], g["ql"], g["ctx"], g["ss"], u, ub,
+                           Lw.x_b)
         ops.gemm_rm(ub.view(M, nb, bw).permute(1, 0, 2), Lw.gates, gates.permute(1, 0, 2), bias=Lw.gates_b)
-        for g in groups:
-            ops.lru_scan(u, gates, yb, Lw.lam, self.state.state[li], g["qs"], g["ql"], g["ctx"], g["ss"], hs,
-                         LRU_DECAY_SCALE)
+        for i, g in enumerate(groups):
+            ops.lru_scan(u, gates, yr, Lw.lam, self.state.state[li], g["qs"], g["ql"], g["ctx"], g["ss"], hs,
+                         LRU_DECAY_SCALE, Lw.y_b, i == 0)
         ops.gemm_rm(hs, Lw.o, d["y"])
 
     def _moe(self, f, Fw, M: int, d: dict):
@@ -154,7 +175,9 @@ class LayeredRunner(RunnerBase):
         tkw = d["tkw"][:M * f.top].view(M, f.top)
         S = f.top + (1 if f.shared_ff else 0)
         o = d["mo_o"][:M * S * self.cfg.width].view(M * S, self.cfg.width)
-        ops.moe_router(d["xb"], Fw.router, Fw.router_b, tki, tkw)
+        z = d["mo_z"][:M * f.experts].view(M, f.experts)
+        ops.gemm_rm(d["xb"], Fw.router, z, bias=Fw.router_b)  # fp32 logits
+        ops.moe_topk(z, tki, tkw)
         ops.moe_grouped(d["xb"], tki, tkw, Fw.gate, Fw.up, Fw.down, Fw.sgate, Fw.sup, Fw.sdown, d["mo_sorted"],
                         d["mo_tile"], d["mo_n"], d["mo_h"], o)
         return o, S

@@ -66,7 +66,14 @@ SMALL = MistralConfig(name="mistral-small", vocab_size=8192, hidden_size=2048, i
 TINY_KV8 = MistralConfig(name="mistral-tiny-kv8", vocab_size=2048, hidden_size=2048, intermediate_size=2048,
                          num_layers=2, num_heads=16, num_kv_heads=8, max_position=4096)
 
-CONFIGS = {c.name: c for c in (MISTRAL_7B_V03, TINY, SMALL, TINY_KV8)}
+# Six layers at the widths of the muderax-mid / muderax-wide benchmark configurations (about the same weights per
+# token and layer): the dense side of bench.py --families.
+MID = MistralConfig(name="mistral-mid", vocab_size=32768, hidden_size=2048, intermediate_size=5632, num_layers=6,
+                    num_heads=16, num_kv_heads=4, max_position=32768)
+WIDE = MistralConfig(name="mistral-wide", vocab_size=32768, hidden_size=4096, intermediate_size=14336, num_layers=6,
+                     num_heads=32, num_kv_heads=8, max_position=32768)
+
+CONFIGS = {c.name: c for c in (MISTRAL_7B_V03, TINY, SMALL, TINY_KV8, MID, WIDE)}
 CONFIGS["mistral-7b"] = MISTRAL_7B_V03
 
 

@@ -250,25 +250,29 @@ def tensor_shapes(cfg: MuderaxConfig) -> dict:
 def init_weights(cfg: MuderaxConfig, seed: int = 0, device="cpu", dtype=torch.bfloat16) -> dict:
     """Random weights in the checkpoint's naming: projections ~ N(0, 1 / fan-in), norm gains near 1, recurrence
     parameters spread so that decays cover fast and slow channels."""
-    g = torch.Generator(device="cpu").manual_seed(seed)
+    dev = torch.device(device)
+    gdev = dev if dev.type == "cuda" else torch.device("cpu")   # large models are drawn on the GPU itself
+    g = torch.Generator(device=gdev).manual_seed(seed)
     out = {}
+
+    def randn(shape):
+        return torch.randn(shape, generator=g, device=gdev)
+
     for name, shape in tensor_shapes(cfg).items():
         leaf = name.rsplit(".", 1)[-1]
         if name == "embed":
-            t = torch.randn(shape, generator=g)
+            t = randn(shape)
         elif leaf in ("norm1", "norm2") or name == "final.norm":
-            t = 1.0 + 0.2 * torch.randn(shape, generator=g)
+            t = 1.0 + 0.2 * randn(shape)
         elif name.endswith("dkv.norm"):
-            t = 1.0 + 0.1 * torch.randn(shape, generator=g)
+            t = 1.0 + 0.1 * randn(shape)
         elif leaf == "lam":
-            t = torch.rand(shape, generator=g) * 4.0 - 3.0
+            t = torch.rand(shape, generator=g, device=gdev) * 4.0 - 3.0
         elif leaf == "b":
-            t = 0.3 * torch.randn(shape, generator=g)
-        elif leaf == "conv":
-            t = torch.randn(shape, generator=g) / math.sqrt(shape[-1])
+            t = 0.3 * randn(shape)
         else:
-            t = torch.randn(shape, generator=g) / math.sqrt(shape[-1])
-        out[name] = t.to(dtype).to(device)
+            t = randn(shape) / math.sqrt(shape[-1])
+        out[name] = t.to(dtype).to(dev)
     return out
 
 
@@ -298,6 +302,6 @@ TINY = _named("muderax-tiny", vocab=512, width=128, n_layers=3, heads=4, dim=32,
 MID = _named("muderax-mid", vocab=32768, width=2048, n_layers=6, heads=16, dim=128, rot_dim=64, vdim=128, rank=512,
              window=2048, rec_width=2560, blocks=10, experts=16, top=2, ff=1408, shared_ff=2816)
 WIDE = _named("muderax-wide", vocab=32768, width=4096, n_layers=6, heads=32, dim=128, rot_dim=64, vdim=128, rank=512,
-              window=4096, rec_width=4096, blocks=16, experts=16, top=2, ff=1792, shared_ff=3584)
+              window=4096, rec_width=4096, blocks=16, experts=16, top=2, ff=3584, shared_ff=7168)
 
 CONFIGS = {c.name: c for c in (TINY, MID, WIDE)}

@@ -67,7 +67,7 @@ def _muderax() -> Family:
         from ..engine.weights import convert_layered
 
         cfg.validate(tp_size)
-        return convert_layered(cfg, X.init_weights(cfg, seed=seed), device=device, dtype=dtype)
+        return convert_layered(cfg, X.init_weights(cfg, seed=seed, device=device), device=device, dtype=dtype)
 
     def load_dir(cfg, path, device, dtype, tp_rank, tp_size):
         from ..engine.weights import load_layered_dir

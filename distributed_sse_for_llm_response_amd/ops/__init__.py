@@ -279,5 +279,5 @@ def kernel_checks(clear: bool = True, raise_on_error: bool = True) -> list:
 
 
 
-from .layers import (conv_state, embed_rows, gemm_rm, latent_attention, latent_flash_ok,  # noqa: E402,F401
-                     latent_kv_write, lru_scan, moe_ffn, moe_grouped, moe_router, scalar_norm)
+from .layers import (conv_state, embed_rows, gemm_rm, latent_attention, latent_flash_ok, latent_flash_part_floats,  # noqa: E402,F401
+                     latent_kv_write, lru_scan, moe_ffn, moe_grouped, moe_router, moe_topk, scalar_norm)

@@ -60,33 +60,51 @@ def latent_flash_ok(dtype, rk: int, dr: int) -> bool:
     return dtype == torch.bfloat16 and rk in (64, 128, 256, 512) and dr % 32 == 0
 
 
+def latent_flash_part_floats(items: int, heads: int, hp: int, nparts: int, rk: int) -> int:
+    """fp32 words of the key-split scratch of latent_attention's MFMA form."""
+    return items * (-(-heads // hp)) * nparts * 16 * (rk + 2)
+
+
 def latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile, rope, out,
-                     window: int, scale: float, qt: int, vt=None, hp: int = 1):
+                     window: int, scale: float, qt: int, vt=None, hp: int = 1, part=None, nparts: int = 1):
     """Sliding-window multi-query attention over the latent cache (folded form), `qt` query rows per work item.
     With vt (transposed latent pages, latent_flash_ok shapes): the MFMA form, qt rows x hp heads = 16 columns per
-    item; without: the row kernel (any sizes, both element types)."""
+    item, the item's keys optionally split over `nparts` partitions (fp32 scratch `part`, latent_flash_part_floats)
+    and merged by a combine kernel; without vt: the row kernel (any sizes, both element types)."""
     if _hip(q):
         torch.ops.dsse.latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile,
-                                        rope, out, window, scale, qt, vt, hp)
+                                        rope, out, window, scale, qt, vt, hp, part, nparts)
     else:
         lref.latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile, rope, out,
                               window, scale, qt, vt)
 
 
-def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b):
-    """Per-channel causal convolution continued from each sequence's slot tail (and the tail's update)."""
+def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias=None):
+    """Per-channel causal convolution continued from each sequence's slot tail (and the tail's update); in_bias is
+    added to every input (the bias of the projection that made `inp`)."""
     if _hip(inp):
-        torch.ops.dsse.conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b)
+        torch.ops.dsse.conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias)
     else:
-        lref.conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b)
+        lref.conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias)
 
 
-def lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, c: float):
-    """Real-gated linear recurrence continued from each sequence's slot state; out = state · y."""
+def lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, c: float, y_bias=None,
+             coeff: bool = True):
+    """Real-gated linear recurrence continued from each sequence's slot state; out = state · gelu(y + y_bias).
+    coeff: turn the gate pre-activations of ALL rows into the recurrence's coefficients first (in place); pass False
+    for a further sequence group of the same step."""
     if _hip(u):
-        torch.ops.dsse.lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, c)
+        torch.ops.dsse.lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, c, y_bias, coeff)
     else:
-        lref.lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, c)
+        lref.lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, c, y_bias, coeff)
+
+
+def moe_topk(logits, topk_idx, topk_w):
+    """The top-k experts of fp32 router logits [M, E] and the softmax over the chosen logits."""
+    if _hip(logits):
+        torch.ops.dsse.moe_topk(logits, topk_idx, topk_w)
+    else:
+        lref.moe_topk(logits, topk_idx, topk_w)
 
 
 def moe_router(x, w, b, topk_idx, topk_w):

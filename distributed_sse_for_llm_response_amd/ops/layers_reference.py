@@ -104,9 +104,10 @@ def latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, wor
             out[row] = (p @ val).to(out.dtype)
 
 
-def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b):
+def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias=None):
     K = taps.shape[1]
     tp = taps.float()
+    ib = 0.0 if in_bias is None else in_bias.float()
     for s in range(q_len.numel()):
         ql = int(q_len[s])
         if ql <= 0:
@@ -114,7 +115,7 @@ def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, 
         r0, slot = int(q_start[s]), int(state_slot[s])
         fresh = int(ctx_len[s]) - ql == 0
         prev = torch.zeros(K - 1, inp.shape[1]) if fresh else tail[slot].clone()
-        seq = torch.cat([prev, inp[r0:r0 + ql]])
+        seq = torch.cat([prev, inp[r0:r0 + ql] + ib])
         y = torch.zeros(ql, inp.shape[1]) if bias is None else bias.float().expand(ql, -1).clone()
         for k in range(K):
             y = y + seq[k:k + ql] * tp[:, k]
@@ -124,10 +125,18 @@ def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, 
             tail[slot] = seq[ql:]
 
 
-def lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, c):
+def lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, c, y_bias=None, coeff=True):
+    """coeff: first turn every row's gate pre-activations [recurrence | input] into the coefficients (a | b) of
+    S = a S + b, in place; then walk each sequence's rows.  y is the gelu branch before its bias and gelu."""
     C = u.shape[1]
     bw = gates.shape[2] // 2
-    sp = torch.nn.functional.softplus(lam.float())
+    if coeff:
+        sp = torch.nn.functional.softplus(lam.float()).view(1, -1, bw)
+        log_a = -c * torch.sigmoid(gates[:, :, :bw]) * sp
+        b = torch.sqrt(-torch.expm1(2.0 * log_a)) * torch.sigmoid(gates[:, :, bw:]) * u.view(u.shape[0], -1, bw)
+        gates[:, :, :bw] = torch.exp(log_a)
+        gates[:, :, bw:] = b
+    yb = 0.0 if y_bias is None else y_bias.float()
     for s in range(q_len.numel()):
         ql = int(q_len[s])
         if ql <= 0:
@@ -136,12 +145,16 @@ def lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, 
         S = torch.zeros(C) if int(ctx_len[s]) - ql == 0 else state[slot].clone()
         for t in range(ql):
             g = gates[r0 + t]
-            r = torch.sigmoid(g[:, :bw]).reshape(C)
-            gi = torch.sigmoid(g[:, bw:]).reshape(C)
-            log_a = -c * r * sp
-            S = torch.exp(log_a) * S + torch.sqrt(-torch.expm1(2.0 * log_a)) * gi * u[r0 + t]
-            out[r0 + t] = (S * y[r0 + t].float()).to(out.dtype)
+            S = g[:, :bw].reshape(C) * S + g[:, bw:].reshape(C)
+            out[r0 + t] = (S * gelu_tanh(y[r0 + t].float() + yb)).to(out.dtype)
         state[slot] = S
+
+
+def moe_topk(logits, topk_idx, topk_w):
+    z = torch.nan_to_num(logits.float(), nan=0.0)
+    val, idx = torch.topk(z, topk_idx.shape[1], dim=-1)
+    topk_idx.copy_(idx.to(torch.int32))
+    topk_w.copy_(torch.softmax(val, dim=-1))
 
 
 def moe_router(x, w, b, topk_idx, topk_w):

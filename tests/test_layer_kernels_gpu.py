@@ -64,6 +64,13 @@ def _case(gpu, H, dn, dr, rk, window, seqs, qt_rows, seed):
     if qt_rows * hp == 16:
         ops.latent_attention(q.to(gpu), q_abs.to(gpu), cache_g, *args, i32(ws), i32(wt), rope.to(gpu), out_flash, window,
                              scale, qt_rows, vt_g, hp)
+    if qt_rows == 1:  # decode: also with the keys split over partitions (more partitions than some items have pages)
+        for nparts in (2, 5, 16):
+            part = torch.full((ops.latent_flash_part_floats(len(ws), H, 16, nparts, rk),), float("nan"), **dev)
+            out_split = torch.zeros_like(out_rows)
+            ops.latent_attention(q.to(gpu), q_abs.to(gpu), cache_g, *args, i32(ws), i32(wt), rope.to(gpu), out_split,
+                                 window, scale, 1, vt_g, 16, part, nparts)
+            assert torch.allclose(out_split.float(), out_flash.float(), atol=2e-2, rtol=2e-2), nparts
     out_ref = torch.zeros(T, H, rk, dtype=torch.float32)
     lref.latent_attention(q, q_abs, cache_g.cpu(), bt, torch.tensor(qs), torch.tensor(ql), torch.tensor(ctx),
                           torch.tensor(ws), torch.tensor(wt), rope, out_ref, window, scale, qt_rows, vt_g.cpu())
@@ -104,14 +111,20 @@ def test_grouped_experts_against_row_kernel(gpu, dtype, M, W, F, Fs, E, top):
     ops.moe_router(x, router, rb, tki, tkw)
     ri, rw = torch.zeros(M, top, dtype=torch.int32), torch.zeros(M, top)
     lref.moe_router(x.cpu(), router.cpu(), rb.cpu(), ri, rw)
+    z = torch.zeros(M, E, device=gpu)
+    ops.gemm_rm(x, router, z, bias=rb)
+    ti2, tw2 = torch.zeros_like(tki), torch.zeros_like(tkw)
+    ops.moe_topk(z, ti2, tw2)
     if dtype == torch.float32:
         assert torch.equal(tki.cpu().sort(-1).values, ri.sort(-1).values)
+        assert torch.equal(ti2.cpu().sort(-1).values, ri.sort(-1).values)
+        assert torch.allclose(tw2.cpu().sort(-1).values, rw.sort(-1).values, atol=1e-5)
     rows = torch.zeros(M, W, device=gpu)
     ops.moe_ffn(x, tki, tkw, gate, up, down, sg, su, sd, rows)
     S = top + (1 if Fs else 0)
-    tiles = -(-M * S // 16) + E + 1
+    tiles = -(-M * S // 64) + E + 2
     o = torch.zeros(M * S, W, device=gpu)
-    ops.moe_grouped(x, tki, tkw, gate, up, down, sg, su, sd, torch.zeros(tiles * 16, dtype=torch.int32, device=gpu),
+    ops.moe_grouped(x, tki, tkw, gate, up, down, sg, su, sd, torch.zeros(tiles * 64, dtype=torch.int32, device=gpu),
                     torch.zeros(tiles, dtype=torch.int32, device=gpu), torch.zeros(1, dtype=torch.int32, device=gpu),
                     torch.zeros(M * S, -(-max(F, Fs) // 8) * 8, dtype=dtype, device=gpu), o)
     ref = torch.zeros(M * S, W)
