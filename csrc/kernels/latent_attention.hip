@@ -295,28 +295,32 @@ __global__ __launch_bounds__(64) void latent_flash_kernel(LatentAttnParams p, co
 // Merge of the key partitions of latent_flash_kernel: per column, M = max of the partitions' maxima,
 // out = sum_z e^(m_z - M) O_z / sum_z e^(m_z - M) l_z.
 __global__ __launch_bounds__(256) void latent_flash_combine_kernel(LatentAttnParams p, int rt, int hp) {
+  // one workgroup per (item, head tile, column)
   const int seq = p.work_seq[blockIdx.x], tile = p.work_tile[blockIdx.x];
   const int ql = p.q_len[seq];
-  if (tile * rt >= ql) return;
+  const int ht = blockIdx.y / 16, col = blockIdx.y % 16;
+  const int off = tile * rt + col / hp, head = ht * hp + col % hp;
+  if (off >= ql || head >= p.H) return;
   const int np = p.nparts;
   const int stride = 16 * (p.rk + 2);
-  const float* base = p.part + ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * np * stride;
-  for (int idx = threadIdx.x; idx < 16 * p.rk; idx += blockDim.x) {
-    const int col = idx / p.rk, d = idx % p.rk;
-    const int off = tile * rt + col / hp, head = blockIdx.y * hp + col % hp;
-    if (off >= ql || head >= p.H) continue;
-    float M = -INFINITY;
-    for (int z = 0; z < np; ++z) M = fmaxf(M, base[z * stride + 16 * p.rk + 2 * col]);
-    float num = 0.f, den = 0.f;
+  const float* base = p.part + ((int64_t)blockIdx.x * (gridDim.y / 16) + ht) * np * stride;
+  const float* ml = base + 16 * p.rk + 2 * col;
+  float M = -INFINITY;
+  for (int z = 0; z < np; ++z) M = fmaxf(M, ml[z * stride]);
+  float den = 0.f;
+  for (int z = 0; z < np; ++z) {
+    const float mz = ml[z * stride];
+    if (mz != -INFINITY) den += expf(mz - M) * ml[z * stride + 1];
+  }
+  const float inv = den > 0.f ? 1.0f / den : 0.0f;
+  bf16* out = reinterpret_cast<bf16*>(p.out) + ((int64_t)(p.q_start[seq] + off) * p.H + head) * p.rk;
+  for (int d = threadIdx.x; d < p.rk; d += blockDim.x) {
+    float num = 0.f;
     for (int z = 0; z < np; ++z) {
-      const float mz = base[z * stride + 16 * p.rk + 2 * col];
-      if (mz == -INFINITY) continue;
-      const float w = expf(mz - M);
-      num += w * base[z * stride + col * p.rk + d];
-      den += w * base[z * stride + 16 * p.rk + 2 * col + 1];
+      const float mz = ml[z * stride];
+      if (mz != -INFINITY) num += expf(mz - M) * base[z * stride + col * p.rk + d];
     }
-    reinterpret_cast<bf16*>(p.out)[((int64_t)(p.q_start[seq] + off) * p.H + head) * p.rk + d] =
-        (bf16)(den > 0.f ? num / den : 0.0f);
+    out[d] = (bf16)(num * inv);
   }
 }
 
@@ -378,6 +382,7 @@ extern "C" hipError_t dsse_latent_flash(int num_work, const dsse::LatentAttnPara
     default: return hipErrorInvalidValue;
   }
   if (np > 1)
-    hipLaunchKernelGGL(dsse::latent_flash_combine_kernel, dim3(num_work, (p->H + hp - 1) / hp), dim3(256), 0, st, *p, rt, hp);
+    hipLaunchKernelGGL(dsse::latent_flash_combine_kernel, dim3(num_work, 16 * ((p->H + hp - 1) / hp)), dim3(256), 0, st, *p, rt,
+                       hp);
   return hipGetLastError();
 }

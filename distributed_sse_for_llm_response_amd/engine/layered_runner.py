@@ -112,6 +112,15 @@ class LayeredRunner(RunnerBase):
         return d
 
     # ------------------------------------------------------------------ layers
+    @staticmethod
+    def _lin(x, w, wt, out) -> None:
+        """out = x · Wᵀ: the engine's tiled-layout GEMMs when the projection was tiled at load (model-sized, aligned
+        shapes: weights.fits_tiled), else the general row-major GEMM."""
+        if wt is not None:
+            ops.gemm_out(x, wt, out)
+        else:
+            ops.gemm_rm(x, w, out)
+
     def _attention(self, li: int, m, Lw, M: int, d: dict, pos, slots, groups: list) -> None:
         H, dn, dr, rk, dv = m.heads, m.dim, m.rot_dim, m.kv_rank, m.vdim
         rope = self._rope[(m.rot, m.rot_dim)]
@@ -121,7 +130,7 @@ class LayeredRunner(RunnerBase):
         qabs = d["qabs"][:M * H * rk].view(M, H, rk)
         lat = d["lat"][:M * H * rk].view(M, H, rk)
         attn = d["attn"][:M * H * dv].view(M, H, dv)
-        ops.gemm_rm(d["xb"], Lw.q, q.view(M, H * (dn + dr)))
+        self._lin(d["xb"], Lw.q, Lw.q_t, q.view(M, H * (dn + dr)))
         ops.gemm_rm(d["xb"], Lw.dkv, ckr)
         vt = self.kv.vt.get(li)
         ops.latent_kv_write(ckr, Lw.dkv_norm, pos, slots, rope, cache, self.cfg.eps, vt)
@@ -141,7 +150,7 @@ class LayeredRunner(RunnerBase):
                 ops.latent_attention(q, qabs, cache, g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"], g["wt"], rope, lat,
                                      m.window, m.scale, g["qt"])
         ops.gemm_rm(lat.permute(1, 0, 2), Lw.uv, attn.permute(1, 0, 2))
-        ops.gemm_rm(attn.view(M, H * dv), Lw.o, d["y"])
+        self._lin(attn.view(M, H * dv), Lw.o, Lw.o_t, d["y"])
 
     def _decode_parts(self, B: int, heads: int, window: int) -> int:
         """Key partitions of the decode attention: enough (item, head tile, partition) waves for the chip, at most one
@@ -158,8 +167,8 @@ class LayeredRunner(RunnerBase):
         gates = d["gates"][:M * 2 * C].view(M, nb, 2 * bw)
         # both input projections leave fp32 without bias: the convolution adds its input's bias, the scan applies
         # the branch's bias and gelu
-        ops.gemm_rm(d["xb"], Lw.y, yr)
-        ops.gemm_rm(d["xb"], Lw.x, ux)
+        self._lin(d["xb"], Lw.y, Lw.y_t, yr)
+        self._lin(d["xb"], Lw.x, Lw.x_t, ux)
         for g in groups:
             ops.conv_state(ux, Lw.conv, Lw.conv_b, self.state.tail[li], g["qs"], g["ql"], g["ctx"], g["ss"], u, ub,
                            Lw.x_b)
@@ -167,7 +176,7 @@ class LayeredRunner(RunnerBase):
         for i, g in enumerate(groups):
             ops.lru_scan(u, gates, yr, Lw.lam, self.state.state[li], g["qs"], g["ql"], g["ctx"], g["ss"], hs,
                          LRU_DECAY_SCALE, Lw.y_b, i == 0)
-        ops.gemm_rm(hs, Lw.o, d["y"])
+        self._lin(hs, Lw.o, Lw.o_t, d["y"])
 
     def _moe(self, f, Fw, M: int, d: dict):
         """Router + grouped experts; returns (per-slot outputs [M * S, W] fp32, S): the norm that follows sums them."""
@@ -204,7 +213,7 @@ class LayeredRunner(RunnerBase):
         """rows: fp32 stream rows (not normed yet) -> final one-number norm -> head GEMM."""
         xn = torch.empty(rows.shape, device=rows.device, dtype=self.dtype)
         ops.scalar_norm(None, self.w.final_norm, rows.contiguous(), xn, self.cfg.eps)
-        ops.gemm_rm(xn, self.w.head, logits)
+        self._lin(xn, self.w.head, self.w.head_t, logits)
 
     # ------------------------------------------------------------------ decode
     def _decode_group(self, B: int) -> dict:
@@ -222,7 +231,7 @@ class LayeredRunner(RunnerBase):
         self._layers(B, d, self.ids[r], self.positions[r], self.slots[r], [self._decode_group(B)])
         xn = self._dec["xb"][:B]
         ops.scalar_norm(None, self.w.final_norm, d["resid"], xn, self.cfg.eps)
-        ops.gemm_rm(xn, self.w.head, self.logits[r])
+        self._lin(xn, self.w.head, self.w.head_t, self.logits[r])
         self._sample_commit(B)
         ops.ring_advance(self.ring_counter)
 

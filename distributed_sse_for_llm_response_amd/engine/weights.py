@@ -206,6 +206,8 @@ class LatentAttentionWeights:
     uk_t: torch.Tensor       # [H, rk, dn]: the key up-projection transposed per head (folds into the query)
     uv: torch.Tensor         # [H, dv, rk]
     o: torch.Tensor          # [W, H dv]
+    q_t: torch.Tensor = None  # q / o in the tiled layout (tile_weight) when their shapes fit the engine's tiled-layout
+    o_t: torch.Tensor = None  # GEMMs; the row-major tensor is then dropped (None)
 
 
 @dataclass
@@ -220,6 +222,9 @@ class RglruWeights:
     gates_b: torch.Tensor    # [blocks, 2 bw]
     lam: torch.Tensor        # [C]
     o: torch.Tensor          # [W, C]
+    y_t: torch.Tensor = None  # y / x / o in the tiled layout when their shapes fit (row-major then None)
+    x_t: torch.Tensor = None
+    o_t: torch.Tensor = None
 
 
 @dataclass
@@ -252,6 +257,7 @@ class LayeredWeights:
     dtype: torch.dtype = torch.bfloat16
     tp_rank: int = 0
     tp_size: int = 1
+    head_t: torch.Tensor = None  # the head in the tiled layout when its shape fits (head then None)
 
     @property
     def vocab_local(self) -> int:
@@ -270,7 +276,27 @@ class LayeredWeights:
             for obj in (L, L.mix, L.mlp):
                 if obj is not None:
                     n += sum(t.numel() * t.element_size() for t in vars(obj).values() if isinstance(t, torch.Tensor))
-        return n + sum(t.numel() * t.element_size() for t in (self.embed, self.final_norm, self.head))
+        return n + sum(t.numel() * t.element_size() for t in (self.embed, self.final_norm, self.head, self.head_t)
+                       if t is not None)
+
+
+TILED_MIN = 1024  # smallest N and K that go to the tiled-layout GEMMs
+
+
+def fits_tiled(w: torch.Tensor) -> bool:
+    """A bf16 [N, K] projection that the engine's tiled-layout GEMMs (ops.gemm_out: skinny / stream / wide / tiled /
+    pipe kernels, picked per row count) serve at every row count: N % 128 == 0, K % 512 == 0, model-sized."""
+    N, K = w.shape
+    return (w.dtype == torch.bfloat16 and N % 128 == 0 and K % 512 == 0 and N >= TILED_MIN and K >= TILED_MIN
+            and N * K * 2 < 2 ** 31)
+
+
+def _tile_fields(obj, names) -> None:
+    for n in names:
+        w = getattr(obj, n)
+        if w is not None and w.dim() == 2 and fits_tiled(w):
+            setattr(obj, n + "_t", tile_weight(w))
+            setattr(obj, n, None)
 
 
 @torch.no_grad()
@@ -307,6 +333,7 @@ def convert_layered(cfg, tensors: dict, device="cpu", dtype=torch.bfloat16) -> L
                 conv_b=t(p + "mix.conv.b"), gates=torch.cat([t(p + "mix.ra"), t(p + "mix.ri")], dim=1).contiguous(),
                 gates_b=torch.cat([t(p + "mix.ra.b"), t(p + "mix.ri.b")], dim=1).contiguous(), lam=t(p + "mix.lam"),
                 o=t(p + "mix.o"))
+        _tile_fields(mix, ("q", "o") if L.kind == "latent_attention" else ("y", "x", "o"))
         layer = LayeredLayer(norm1=one(p + "norm1"), mix=mix)
         if L.mlp is not None:
             f = L.mlp
@@ -318,8 +345,10 @@ def convert_layered(cfg, tensors: dict, device="cpu", dtype=torch.bfloat16) -> L
                 layer.mlp.sgate, layer.mlp.sup, layer.mlp.sdown = (t(f"{p}mlp.shared.{leaf}")
                                                                    for leaf in ("gate", "up", "down"))
         own[i] = layer
-    return LayeredWeights(cfg=cfg, embed=t("embed"), layers=[own[L.weights_of] for L in cfg.layers],
-                          final_norm=one("final.norm"), head=t("head"), dtype=dtype)
+    out = LayeredWeights(cfg=cfg, embed=t("embed"), layers=[own[L.weights_of] for L in cfg.layers],
+                         final_norm=one("final.norm"), head=t("head"), dtype=dtype)
+    _tile_fields(out, ("head",))
+    return out
 
 
 def load_layered_dir(cfg, path: str, device="cpu", dtype=torch.bfloat16) -> LayeredWeights:

@@ -133,3 +133,24 @@ def test_grouped_experts_against_row_kernel(gpu, dtype, M, W, F, Fs, E, top):
     tol = 1e-4 if dtype == torch.float32 else 3e-2
     assert torch.allclose(o.cpu(), ref, atol=tol, rtol=tol), float((o.cpu() - ref).abs().max())
     assert torch.allclose(o.view(M, S, W).sum(1).cpu(), rows.cpu(), atol=tol, rtol=tol)
+
+
+@pytest.mark.parametrize("N,K", [(1024, 1024), (3072, 2048), (2048, 2560)])
+def test_tiled_dispatch_matches_row_major(gpu, N, K):
+    """Projections that fit the tiled-layout GEMMs (weights.fits_tiled) against the general row-major GEMM, for the row
+    counts of decode buckets, mixed steps and prompt passes, with bf16 and fp32 output."""
+    from distributed_sse_for_llm_response_amd.engine.weights import fits_tiled
+    from distributed_sse_for_llm_response_amd.ops.reference import tile_weight
+
+    g = torch.Generator().manual_seed(N + K)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).to(gpu)
+    assert fits_tiled(w)
+    wt = tile_weight(w)
+    for M in (1, 3, 16, 17, 64, 65, 130, 257, 600, 1113):
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(gpu)
+        for dt in (torch.float32, torch.bfloat16):
+            a, b = torch.zeros(M, N, dtype=dt, device=gpu), torch.zeros(M, N, dtype=dt, device=gpu)
+            ops.gemm_rm(x, w, a)
+            ops.gemm_out(x, wt, b)
+            tol = 2e-3 if dt == torch.float32 else 2e-2
+            assert torch.allclose(a.float(), b.float(), atol=tol, rtol=tol), (M, dt, float((a.float() - b.float()).abs().max()))

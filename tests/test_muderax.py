@@ -332,6 +332,8 @@ def test_long_decoding(device):
     ("sizes that vector loads like", config([with_mlp(att(heads=4, dim=32, rot_dim=16, vdim=24, kv_rank=64, window=20),
                                                       moe(8, 2, 40, 48)), with_mlp(rec(width=96, blocks=4, conv=4),
                                                                                    moe(8, 2, 40, 48))], width=64, vocab=96)),
+    ("projections on the tiled-layout GEMMs", config([att(heads=8, dim=96, rot_dim=32, vdim=128, kv_rank=64, window=30),
+                                                      rec(width=1024, blocks=4, conv=4)], width=1024, vocab=1024)),
     ("wide rows", config([att(heads=2, dim=8, rot_dim=4, vdim=8, kv_rank=300, window=17),
                           with_mlp(rec(width=600, blocks=2, conv=4), moe(3, 2, 70, 0))], width=520, vocab=300)),
 ])
