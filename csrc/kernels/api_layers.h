@@ -159,11 +159,10 @@ hipError_t dsse_gemm_rm(const dsse::GemmRmParams* p, hipStream_t st);
 hipError_t dsse_scalar_norm(const dsse::ScalarNormParams* p, hipStream_t st);
 hipError_t dsse_embed_rows(int M, int W, int vocab, const int* ids, const void* embed, float* resid, void* xb, int f32,
                            hipStream_t st);
-hipError_t dsse_latent_kv_write(const dsse::LatentKvWriteParams* p, hipStream_t st);
+hipError_t dsse_latent_kv_write(const dsse::LatentKvWriteParams* p, void* vt, hipStream_t st);  // vt: see below, or null
 hipError_t dsse_latent_attention(int num_work, const dsse::LatentAttnParams* p, hipStream_t st);
 // transposed latent pages vt [pages, rk, kBS] (keys permuted inside a page) for the MFMA form, and that form itself
 // (bf16, rk in {64, 128, 256, 512}, dr % 32 == 0; 16 columns = rt rows x hp heads per work item)
-hipError_t dsse_latent_vt_write(const dsse::LatentKvWriteParams* p, void* vt, hipStream_t st);
 hipError_t dsse_latent_flash(int num_work, const dsse::LatentAttnParams* p, const void* vt, int rt, int hp,
                              hipStream_t st);
 hipError_t dsse_conv_state(const dsse::ConvStateParams* p, hipStream_t st);

@@ -155,14 +155,15 @@ void latent_kv_write(const Tensor& ckr, const Tensor& norm_w, const Tensor& posi
   p.num_slots = (int)(cache.size(0) * dsse::kBS);
   p.eps = (float)eps;
   p.f32 = elem(cache, "cache");
-  DSSE_CHECK_HIP(dsse_latent_kv_write(&p, cur_stream()));
+  void* vtp = nullptr;
   if (vt.has_value()) {
     gpu(*vt, "vt");
     same(cache, *vt, "vt");
     TORCH_CHECK(vt->dim() == 3 && vt->size(0) == cache.size(0) && vt->size(1) == rk && vt->size(2) == dsse::kBS,
                 "vt must be [pages, rk, 32]");
-    DSSE_CHECK_HIP(dsse_latent_vt_write(&p, vt->data_ptr(), cur_stream()));
+    vtp = vt->data_ptr();
   }
+  DSSE_CHECK_HIP(dsse_latent_kv_write(&p, vtp, cur_stream()));
 }
 
 void latent_attention(const Tensor& q, const Tensor& q_abs, const Tensor& cache, const Tensor& block_tables,

@@ -7,6 +7,7 @@
 // kernel is multi-query attention with key width rk + dr and value width rk.
 //
 //   latent_kv_write   c = rms-norm(down-projection[:rk]) * w, kr = rot(down-projection[rk:]) -> cache row of the token
+//                     (and c once more into the transposed page that the MFMA form reads its values from)
 //   latent_attention  generic row kernel (any element type, any sizes): one workgroup per (query tile, head), the
 //                     tile's rows one after the other; keys max(0, pos - window + 1) .. pos through the block table,
 //                     256 keys per pass (one key per thread for the scores, one latent coordinate per thread for the
@@ -39,7 +40,7 @@ DEV float block_reduce_max(float v, float* red) {
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void latent_kv_write_kernel(LatentKvWriteParams p) {
+__global__ __launch_bounds__(256) void latent_kv_write_kernel(LatentKvWriteParams p, T* __restrict__ vt) {
   __shared__ float red[4];
   const int row = blockIdx.x;
   const int slot = p.slots[row];
@@ -52,7 +53,15 @@ __global__ __launch_bounds__(256) void latent_kv_write_kernel(LatentKvWriteParam
   ss = block_reduce_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)p.rk + p.eps);
   const T* nw = reinterpret_cast<const T*>(p.norm_w);
-  for (int d = threadIdx.x; d < p.rk; d += blockDim.x) dst[d] = (T)(src[d] * inv * (float)nw[d]);
+  // vt (optional): the latent once more in the transposed page of the MFMA attention form, key order of that form
+  const int off = slot % kBS;
+  T* vdst = vt ? vt + (int64_t)(slot / kBS) * p.rk * kBS + (((off & 15) >> 2) * 8 + ((off >> 4) & 1) * 4 + (off & 3))
+               : nullptr;
+  for (int d = threadIdx.x; d < p.rk; d += blockDim.x) {
+    const T v = (T)(src[d] * inv * (float)nw[d]);
+    dst[d] = v;
+    if (vdst) vdst[(int64_t)d * kBS] = v;
+  }
   int pos = p.positions[row];
   pos = pos < 0 ? 0 : (pos >= p.rope_len ? p.rope_len - 1 : pos);
   const float2* cs = p.rope + (int64_t)pos * (p.dr / 2);
@@ -324,24 +333,14 @@ __global__ __launch_bounds__(256) void latent_flash_combine_kernel(LatentAttnPar
   }
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void latent_vt_write_kernel(LatentKvWriteParams p, T* __restrict__ vt) {
-  // after latent_kv_write: copy the token's normed latent from its cache row into the transposed page
-  const int row = blockIdx.x;
-  const int slot = p.slots[row];
-  if (slot < 0 || slot >= p.num_slots) return;
-  const int blk = slot / kBS, off = slot % kBS;
-  const int at = ((off & 15) >> 2) * 8 + ((off >> 4) & 1) * 4 + (off & 3);
-  const T* src = reinterpret_cast<const T*>(p.cache) + (int64_t)slot * (p.rk + p.dr);
-  for (int d = threadIdx.x; d < p.rk; d += blockDim.x) vt[((int64_t)blk * p.rk + d) * kBS + at] = src[d];
-}
-
 }  // namespace dsse
 
-extern "C" hipError_t dsse_latent_kv_write(const dsse::LatentKvWriteParams* p, hipStream_t st) {
+extern "C" hipError_t dsse_latent_kv_write(const dsse::LatentKvWriteParams* p, void* vt, hipStream_t st) {
   if (p->T <= 0) return hipSuccess;
-  if (p->f32) hipLaunchKernelGGL(dsse::latent_kv_write_kernel<float>, dim3(p->T), dim3(256), 0, st, *p);
-  else hipLaunchKernelGGL(dsse::latent_kv_write_kernel<bf16>, dim3(p->T), dim3(256), 0, st, *p);
+  if (p->f32)
+    hipLaunchKernelGGL(dsse::latent_kv_write_kernel<float>, dim3(p->T), dim3(256), 0, st, *p, reinterpret_cast<float*>(vt));
+  else
+    hipLaunchKernelGGL(dsse::latent_kv_write_kernel<bf16>, dim3(p->T), dim3(256), 0, st, *p, reinterpret_cast<bf16*>(vt));
   return hipGetLastError();
 }
 
@@ -352,15 +351,6 @@ extern "C" hipError_t dsse_latent_attention(int num_work, const dsse::LatentAttn
   dim3 grid(num_work, p->H);
   if (p->f32) hipLaunchKernelGGL(dsse::latent_attention_rows_kernel<float>, grid, dim3(256), lds, st, *p);
   else hipLaunchKernelGGL(dsse::latent_attention_rows_kernel<bf16>, grid, dim3(256), lds, st, *p);
-  return hipGetLastError();
-}
-
-extern "C" hipError_t dsse_latent_vt_write(const dsse::LatentKvWriteParams* p, void* vt, hipStream_t st) {
-  if (p->T <= 0) return hipSuccess;
-  if (p->f32)
-    hipLaunchKernelGGL(dsse::latent_vt_write_kernel<float>, dim3(p->T), dim3(256), 0, st, *p, reinterpret_cast<float*>(vt));
-  else
-    hipLaunchKernelGGL(dsse::latent_vt_write_kernel<bf16>, dim3(p->T), dim3(256), 0, st, *p, reinterpret_cast<bf16*>(vt));
   return hipGetLastError();
 }
 

@@ -193,15 +193,36 @@ __global__ __launch_bounds__(256) void moe_align_kernel(MoeGroupedParams p) {
   }
 }
 
+// Both expert GEMMs: a workgroup owns 16 output columns of one 64-row tile; its four waves split the K axis (k-steps
+// w, w + 4, ...) and meet in LDS, where wave i finishes the tile's i-th 16-row sub-tile.  Sixteen columns per workgroup
+// give a decode step (17 tiles or so) thousands of workgroups to hide the weight stream's latency with.
+DEV void reduce4(f32x4 (&acc)[4], float* red, int wave, int lane) {
+  // red [wave][sub][reg][lane]; afterwards acc[wave] of every wave holds the sum over the four waves of sub-tile `wave`
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) red[((wave * 4 + i) * 4 + j) * 64 + lane] = acc[i][j];
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) v += red[((w * 4 + wave) * 4 + j) * 64 + lane];
+    acc[0][j] = v;
+  }
+  __syncthreads();
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(MoeGroupedParams p) {
   using F = Frag<T>;
+  __shared__ float red[4 * 4 * 4 * 64];
   const int t = blockIdx.y;
   if (t >= *p.num_tiles) return;
   const int e = p.tile_expert[t];
   const bool sh = e >= p.E;
   const int Fe = sh ? p.Fs : p.F;
-  if ((int)blockIdx.x * 64 >= Fe) return;
+  if ((int)blockIdx.x * 16 >= Fe) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
   const T* gate = sh ? reinterpret_cast<const T*>(p.sgate) : reinterpret_cast<const T*>(p.gate) + (int64_t)e * p.F * p.W;
   const T* up = sh ? reinterpret_cast<const T*>(p.sup) : reinterpret_cast<const T*>(p.up) + (int64_t)e * p.F * p.W;
@@ -216,7 +237,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(MoeGroupedParams p) {
     xv[i] = id >= 0;
     xr[i] = reinterpret_cast<const T*>(p.x) + (int64_t)(xv[i] ? id / p.S : 0) * p.W;
   }
-  const int f = blockIdx.x * 64 + wave * 16 + r;
+  const int f = blockIdx.x * 16 + r;
   const bool fv = f < Fe;
   const T* gr = gate + (int64_t)(fv ? f : 0) * p.W;
   const T* ur = up + (int64_t)(fv ? f : 0) * p.W;
@@ -224,7 +245,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(MoeGroupedParams p) {
   f32x4 ag[4], au[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) ag[i] = au[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < p.W; k0 += F::KS) {
+  for (int k0 = wave * F::KS; k0 < p.W; k0 += 4 * F::KS) {
     const int k = k0 + F::PER * g;
     const typename F::V bg = load_frag<T>(gr, k, p.W, fv, vec), bu = load_frag<T>(ur, k, p.W, fv, vec);
 #pragma unroll
@@ -235,23 +256,22 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(MoeGroupedParams p) {
       au[i] = mma(a, bu, au[i]);
     }
   }
-  if (!fv) return;
+  reduce4(ag, red, wave, lane);
+  reduce4(au, red, wave, lane);
+  if (!fv || !live[wave]) return;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    if (!live[i]) continue;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int id2 = ids[16 * i + 4 * g + j];
-      if (id2 < 0) continue;
-      const float gv = ag[i][j];
-      reinterpret_cast<T*>(p.h)[(int64_t)id2 * p.ldh + f] = (T)(gv / (1.0f + expf(-gv)) * au[i][j]);
-    }
+  for (int j = 0; j < 4; ++j) {
+    const int id2 = ids[16 * wave + 4 * g + j];
+    if (id2 < 0) continue;
+    const float gv = ag[0][j];
+    reinterpret_cast<T*>(p.h)[(int64_t)id2 * p.ldh + f] = (T)(gv / (1.0f + expf(-gv)) * au[0][j]);
   }
 }
 
 template <typename T>
 __global__ __launch_bounds__(256) void moe_down_kernel(MoeGroupedParams p) {
   using F = Frag<T>;
+  __shared__ float red[4 * 4 * 4 * 64];
   const int t = blockIdx.y;
   if (t >= *p.num_tiles) return;
   const int e = p.tile_expert[t];
@@ -269,14 +289,14 @@ __global__ __launch_bounds__(256) void moe_down_kernel(MoeGroupedParams p) {
     hv[i] = id >= 0;
     hr[i] = reinterpret_cast<const T*>(p.h) + (int64_t)(hv[i] ? id : 0) * p.ldh;
   }
-  const int d = blockIdx.x * 64 + wave * 16 + r;
+  const int d = blockIdx.x * 16 + r;
   const bool dv = d < p.W;
   const T* dr = down + (int64_t)(dv ? d : 0) * Fe;
   const bool vech = p.vec_h != 0, vecd = p.vec_h != 0 && Fe % F::PER == 0;
   f32x4 acc[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < Fe; k0 += F::KS) {
+  for (int k0 = wave * F::KS; k0 < Fe; k0 += 4 * F::KS) {
     const int k = k0 + F::PER * g;
     const typename F::V b = load_frag<T>(dr, k, Fe, dv, vecd);
 #pragma unroll
@@ -285,18 +305,15 @@ __global__ __launch_bounds__(256) void moe_down_kernel(MoeGroupedParams p) {
       acc[i] = mma(load_frag<T>(hr[i], k, Fe, hv[i], vech), b, acc[i]);
     }
   }
-  if (!dv) return;
+  reduce4(acc, red, wave, lane);
+  if (!dv || !live[wave]) return;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    if (!live[i]) continue;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int id2 = ids[16 * i + 4 * g + j];
-      if (id2 < 0) continue;
-      const int row = id2 / p.S, k = id2 % p.S;
-      const float wgt = k < p.top ? p.topk_w[row * p.top + k] : 1.0f;
-      p.o[(int64_t)id2 * p.W + d] = wgt * acc[i][j];
-    }
+  for (int j = 0; j < 4; ++j) {
+    const int id2 = ids[16 * wave + 4 * g + j];
+    if (id2 < 0) continue;
+    const int row = id2 / p.S, k = id2 % p.S;
+    const float wgt = k < p.top ? p.topk_w[row * p.top + k] : 1.0f;
+    p.o[(int64_t)id2 * p.W + d] = wgt * acc[0][j];
   }
 }
 
@@ -326,7 +343,7 @@ extern "C" hipError_t dsse_moe_grouped(const dsse::MoeGroupedParams* p, hipStrea
   const int NE = p->E + (p->S > p->top ? 1 : 0);
   hipLaunchKernelGGL(dsse::moe_align_kernel, dim3(1), dim3(256), sizeof(int) * (3 * NE + 1), st, *p);
   const int fmax = p->F > p->Fs ? p->F : p->Fs;
-  dim3 g1((fmax + 63) / 64, p->max_tiles), g2((p->W + 63) / 64, p->max_tiles);
+  dim3 g1((fmax + 15) / 16, p->max_tiles), g2((p->W + 15) / 16, p->max_tiles);
   if (p->f32) {
     hipLaunchKernelGGL(dsse::moe_gate_up_kernel<float>, g1, dim3(256), 0, st, *p);
     hipLaunchKernelGGL(dsse::moe_down_kernel<float>, g2, dim3(256), 0, st, *p);

@@ -38,7 +38,8 @@ from .weights import LayeredWeights
 
 ATTN_ROWS_TILE = 4    # query rows per work item of the row-wise attention kernel (prompt portions)
 FLASH_DECODE_WAVES = 512  # waves a decode attention launch aims for (two per CU)
-FLASH_ROWS_TILE = 16  # query rows per work item of the MFMA attention form (x 16 / rows heads = 16 columns)
+FLASH_ROWS_TILE = 4   # query rows per work item of the MFMA attention form, x 4 heads = 16 columns: a page of keys is
+                      # read once for four heads (16 rows x 1 head re-read it per head: 2-3x the time at 16 heads)
 
 
 class LayeredRunner(RunnerBase):

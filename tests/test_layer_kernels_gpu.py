@@ -79,9 +79,10 @@ def _case(gpu, H, dn, dr, rk, window, seqs, qt_rows, seed):
 
 @pytest.mark.parametrize("H,dn,dr,rk", [(3, 16, 32, 64), (8, 32, 32, 128), (20, 8, 64, 256), (16, 24, 32, 512)])
 @pytest.mark.parametrize("window", [1, 5, 32, 33, 70, 10 ** 6])
-def test_prompt_tiles(gpu, H, dn, dr, rk, window):
+@pytest.mark.parametrize("rows_per_tile", [16, 4, 2])
+def test_prompt_tiles(gpu, H, dn, dr, rk, window, rows_per_tile):
     seqs = [(0, 50), (37, 3), (64, 31), (5, 1), (90, 40)]
-    rows, flash, ref = _case(gpu, H, dn, dr, rk, window, seqs, 16, seed=H + window)
+    rows, flash, ref = _case(gpu, H, dn, dr, rk, window, seqs, rows_per_tile, seed=H + window)
     assert torch.allclose(rows, ref, atol=3e-2, rtol=3e-2)
     assert torch.allclose(flash, ref, atol=5e-2, rtol=5e-2), float((flash - ref).abs().max())
 
