@@ -173,20 +173,25 @@ __global__ __launch_bounds__(256) void latent_attention_rows_kernel(LatentAttnPa
 // The last step needs no shuffle because which key a (lane group g, element j) pair of the k axis stands for only has
 // to agree between A and B: the scores of lane group g are keys 4g..4g+3 of both 16-key halves, so the transposed page
 // stores key k at position 8 ((k & 15) >> 2) + 4 (k >> 4) + (k & 3) (the dense KV cache's V pages use the same order).
+// A workgroup is up to four such waves: the head tiles of the SAME rows, which walk the same pages at the same time and
+// so share them in the CU's L1 instead of each pulling the whole window from L2 (the launch is L2-bound otherwise).
 template <int NT>  // rk / 16 value tiles
-__global__ __launch_bounds__(64) void latent_flash_kernel(LatentAttnParams p, const bf16* __restrict__ vt, int rt, int hp) {
+__global__ __launch_bounds__(256) void latent_flash_kernel(LatentAttnParams p, const bf16* __restrict__ vt, int rt, int hp,
+                                                           int head_tiles) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   const int D = p.rk + p.dr;
   const int ldq = D + 8;  // bf16 elements per LDS row (16 B of padding)
-  bf16* qs = reinterpret_cast<bf16*>(smem_raw);  // [16][ldq]
-  const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
+  const int wave = threadIdx.x >> 6;
+  const int hy = blockIdx.y * (blockDim.x >> 6) + wave;  // this wave's head tile
+  bf16* qs = reinterpret_cast<bf16*>(smem_raw) + wave * 16 * ldq;  // [16][ldq] per wave
+  const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
   const int seq = p.work_seq[blockIdx.x], tile = p.work_tile[blockIdx.x];
   const int ql = p.q_len[seq];
   if (tile * rt >= ql) return;
   const int q0 = p.q_start[seq], pos0 = p.ctx_len[seq] - ql;
   // this lane's column
-  const int c_off = tile * rt + r / hp, c_head = blockIdx.y * hp + r % hp;
-  const bool c_ok = c_off < ql && c_head < p.H;
+  const int c_off = tile * rt + r / hp, c_head = hy * hp + r % hp;
+  const bool c_ok = c_off < ql && c_head < p.H && hy < head_tiles;
   const int c_pos = c_ok ? pos0 + c_off : -1;
   const int64_t c_row = q0 + (c_ok ? c_off : 0);
   // stage the 16 query vectors: lane group g fills coordinates g, g + 4, ... (in chunks of 8) of column r
@@ -214,6 +219,7 @@ __global__ __launch_bounds__(64) void latent_flash_kernel(LatentAttnParams p, co
     }
   }
   __syncthreads();
+  if (hy >= head_tiles) return;
   // key range of the tile: from the first row's window start to the last row's position
   const int last_off = (tile * rt + rt - 1 < ql ? tile * rt + rt - 1 : ql - 1);
   const int hi = pos0 + last_off;
@@ -238,11 +244,31 @@ __global__ __launch_bounds__(64) void latent_flash_kernel(LatentAttnParams p, co
     blk = (unsigned)blk < (unsigned)p.num_blocks ? blk : 0;
     const bf16* krow0 = rows + ((int64_t)blk * kBS + r) * D + 8 * g;        // key r of the page's first half
     const bf16* krow1 = krow0 + (int64_t)16 * D;                             // key 16 + r
+    // the page's value fragments are requested first: they arrive while the scores are computed (a single wave per
+    // SIMD has nothing else to hide their latency behind)
+    const bf16* vrow = vt + ((int64_t)blk * p.rk + r) * kBS + 8 * g;  // dim r of value tile 0, positions 8g..8g+7
+    bf16x8 vf[NT];
+#pragma unroll
+    for (int n = 0; n < NT; ++n) vf[n] = ld_bf16x8(vrow + (int64_t)n * 16 * kBS);
     f32x4 s0 = f32x4{0.f, 0.f, 0.f, 0.f}, s1 = s0;
-    for (int s = 0; s < nks; ++s) {
-      const bf16x8 b = *reinterpret_cast<const bf16x8*>(qs + r * ldq + 32 * s + 8 * g);
-      s0 = mfma16x16x32(ld_bf16x8(krow0 + 32 * s), b, s0);
-      s1 = mfma16x16x32(ld_bf16x8(krow1 + 32 * s), b, s1);
+    // six k-steps at a time: their twelve key loads are issued before the first MFMA needs one (a single wave per
+    // work item has nothing else to hide the load latency behind)
+    for (int sb = 0; sb < nks; sb += 6) {
+      bf16x8 ka[6], kb[6], qb[6];
+#pragma unroll
+      for (int u = 0; u < 6; ++u) {
+        const int s = sb + u < nks ? sb + u : nks - 1;  // past the end: a valid address, the product is skipped
+        ka[u] = ld_bf16x8(krow0 + 32 * s);
+        kb[u] = ld_bf16x8(krow1 + 32 * s);
+        qb[u] = *reinterpret_cast<const bf16x8*>(qs + r * ldq + 32 * s + 8 * g);
+      }
+#pragma unroll
+      for (int u = 0; u < 6; ++u) {
+        if (sb + u < nks) {
+          s0 = mfma16x16x32(ka[u], qb[u], s0);
+          s1 = mfma16x16x32(kb[u], qb[u], s1);
+        }
+      }
     }
     // lane (r, g): column r, keys pg * 32 + 4 g + i (s0) and + 16 (s1)
     float sv[8];
@@ -267,17 +293,16 @@ __global__ __launch_bounds__(64) void latent_flash_kernel(LatentAttnParams p, co
     }
     l = l * corr + rows4_sum(ps);
     m = mn;
-    const bf16* vrow = vt + ((int64_t)blk * p.rk + r) * kBS + 8 * g;  // dim r of value tile 0, positions 8g..8g+7
 #pragma unroll
     for (int n = 0; n < NT; ++n) {
       f32x4 o = O[n];
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[i] *= corr;
-      O[n] = mfma16x16x32(ld_bf16x8(vrow + (int64_t)n * 16 * kBS), pf, o);
+      O[n] = mfma16x16x32(vf[n], pf, o);
     }
   }
   if (np > 1) {
-    float* po = p.part + (((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * np + blockIdx.z) * (16 * (p.rk + 2));
+    float* po = p.part + (((int64_t)blockIdx.x * head_tiles + hy) * np + blockIdx.z) * (16 * (p.rk + 2));
 #pragma unroll
     for (int n = 0; n < NT; ++n)
 #pragma unroll
@@ -359,16 +384,18 @@ extern "C" hipError_t dsse_latent_flash(int num_work, const dsse::LatentAttnPara
                                         hipStream_t st) {
   if (num_work <= 0) return hipSuccess;
   if (p->f32 || rt * hp != 16 || p->rk % 32 || p->dr % 32) return hipErrorInvalidValue;
-  const size_t lds = 16 * (size_t)(p->rk + p->dr + 8) * sizeof(bf16);
   const int np = p->nparts > 1 ? p->nparts : 1;
   if (np > 1 && !p->part) return hipErrorInvalidValue;
-  dim3 grid(num_work, (p->H + hp - 1) / hp, np);
+  const int gy = (p->H + hp - 1) / hp;          // head tiles
+  const int wy = gy < 4 ? gy : 4;               // of them, waves per workgroup
+  const size_t lds = wy * 16 * (size_t)(p->rk + p->dr + 8) * sizeof(bf16);
+  dim3 grid(num_work, (gy + wy - 1) / wy, np), block(64 * wy);
   const bf16* v = reinterpret_cast<const bf16*>(vt);
   switch (p->rk / 16) {
-    case 4: hipLaunchKernelGGL(dsse::latent_flash_kernel<4>, grid, dim3(64), lds, st, *p, v, rt, hp); break;
-    case 8: hipLaunchKernelGGL(dsse::latent_flash_kernel<8>, grid, dim3(64), lds, st, *p, v, rt, hp); break;
-    case 16: hipLaunchKernelGGL(dsse::latent_flash_kernel<16>, grid, dim3(64), lds, st, *p, v, rt, hp); break;
-    case 32: hipLaunchKernelGGL(dsse::latent_flash_kernel<32>, grid, dim3(64), lds, st, *p, v, rt, hp); break;
+    case 4: hipLaunchKernelGGL(dsse::latent_flash_kernel<4>, grid, block, lds, st, *p, v, rt, hp, gy); break;
+    case 8: hipLaunchKernelGGL(dsse::latent_flash_kernel<8>, grid, block, lds, st, *p, v, rt, hp, gy); break;
+    case 16: hipLaunchKernelGGL(dsse::latent_flash_kernel<16>, grid, block, lds, st, *p, v, rt, hp, gy); break;
+    case 32: hipLaunchKernelGGL(dsse::latent_flash_kernel<32>, grid, block, lds, st, *p, v, rt, hp, gy); break;
     default: return hipErrorInvalidValue;
   }
   if (np > 1)
