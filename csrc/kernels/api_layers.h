@@ -74,7 +74,7 @@ struct LatentAttnParams {
 
 struct ConvStateParams {
   const float* in;       // [T, C] fp32
-  const void* taps;      // [C, K] (last column = the current token)
+  const void* taps;      // [C, K]; taps[c][K - 1] weighs the newest input
   const void* bias;      // [C]
   const void* in_bias;   // [C] or null: added to every input (the input projection's bias; tails hold biased inputs)
   float* tail;           // [slots, K - 1, C] last K - 1 inputs of each sequence

@@ -1,4 +1,4 @@
-// Routed mixture of experts: router (fp32 logits, top-k, softmax over the chosen logits only) and the token-major
+// Routed mixture of experts: router (fp32 logits, the k largest, a softmax among those k) and the token-major
 // expert feed-forward (each row walks its chosen experts and the always-on shared expert).
 //
 //   moe_router   one wave per row: logits z[e] = w[e] . x + b[e] in fp32 (lanes split the width, wave reduction), then

@@ -2,7 +2,7 @@
 // the engine's per-sequence state slots.
 //
 //   conv_state   out[t, c] = b[c] + sum_k taps[c, k] * in[t - (K - 1) + k, c]; inputs before the step's first row come
-//                from the slot's tail (the last K - 1 inputs of the sequence), zeros before the sequence's start.  The
+//                from the slot's tail (the last K - 1 inputs of the sequence), an empty (zero) history at position 0.  The
 //                tail is rewritten with the step's last K - 1 inputs (shifted in place when the step is shorter).
 //   lru_scan     r = sigmoid(gate_r), i = sigmoid(gate_i), log a = -c r softplus(lam), S = a S + sqrt(1 - a^2) i u,
 //                out = S * y.  The state S is fp32 and lives in the sequence's slot; a sequence's first step starts from

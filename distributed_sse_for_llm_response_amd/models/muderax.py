@@ -3,8 +3,8 @@
 Every layer is ``x += n1(mixer(x)); x += n2(ffn(x))`` on an fp32 residual stream, where the sublayers read the stream
 itself and ``n`` is a one-number RMS norm on the sublayer's OUTPUT.  Mixers:
 
-* ``latent_attention`` -- attention whose keys and values are up-projected from a cached low-rank latent (plus one
-  rotated key part shared by all heads), sliding-window mask, interleaved rotary pairs with YaRN frequency scaling;
+* ``latent_attention`` -- attention whose keys and values are up-projected from a cached low-rank latent (plus a single
+  rotated key slice that every head uses), sliding-window mask, interleaved rotary pairs with YaRN frequency scaling;
 * ``rglru`` -- a gelu branch times a real-gated linear recurrence over a short causal convolution, gates block-diagonal.
 
 The feed-forward is a routed mixture of gated-SiLU experts (softmax over the chosen router logits) plus an always-on
@@ -150,6 +150,12 @@ class MuderaxConfig:
                 mlp = MoeSpec(experts=int(f["router"]["experts"]), top=int(f["router"]["top"]),
                               ff=int(f["expert"]["ff"]), shared_ff=int(sh.get("ff", 0)))
             layers.append(LayerSpec(kind=L["type"], mixer=mixer, mlp=mlp, weights_of=int(L.get("weights_of", i))))
+        for i, L in enumerate(layers):  # a borrower of a borrower uses the tensors of the layer that owns them
+            j, hops = L.weights_of, 0
+            while layers[j].weights_of != j and hops < len(layers):
+                j, hops = layers[j].weights_of, hops + 1
+            if j != L.weights_of:
+                layers[i] = LayerSpec(kind=L.kind, mixer=L.mixer, mlp=L.mlp, weights_of=j)
         cfg = cls(vocab_size=int(d["vocab"]), width=int(d["width"]), eps=float(d["norm"]["eps"]),
                   layers=tuple(layers), name=name, raw=d)
         cfg.validate()
@@ -187,9 +193,11 @@ class MuderaxConfig:
             raise ValueError("Muderax runs on one GPU per replica (no tensor-parallel sharding of its layers)")
         for i, L in enumerate(self.layers):
             src = self.layers[L.weights_of]
-            if L.weights_of != i and (src.weights_of != L.weights_of or (src.kind, src.mixer, src.mlp) !=
-                                      (L.kind, L.mixer, L.mlp)):
-                raise ValueError(f"layer {i} borrows weights of layer {L.weights_of}, which differs or borrows itself")
+            # a borrower runs with its OWN constants (window, scale, rotation) on the lender's tensors: the kinds and
+            # every tensor shape must agree
+            if L.weights_of != i and (src.weights_of != L.weights_of or src.kind != L.kind or
+                                      _shape_key(src) != _shape_key(L)):
+                raise ValueError(f"layer {i} borrows the weights of layer {L.weights_of}, whose tensors differ in shape")
             m = L.mixer
             if L.kind == "latent_attention":
                 if m.rot_dim % 2 or m.rot.dims % 2 or m.rot.dims > m.rot_dim or m.kv_rank > 1024 or m.window < 1:
@@ -209,6 +217,13 @@ class MuderaxConfig:
     def cache_bytes_per_token(self, elem_bytes: int = 2) -> int:
         return sum((L.mixer.kv_rank + L.mixer.rot_dim) * elem_bytes for L in self.layers
                    if L.kind == "latent_attention")
+
+
+def _shape_key(L: LayerSpec) -> tuple:
+    m = L.mixer
+    mix = (m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank) if L.kind == "latent_attention" else (m.width, m.blocks, m.conv)
+    f = L.mlp
+    return mix, (None if f is None else (f.experts, f.ff, f.shared_ff))
 
 
 def layer_tensor_shapes(cfg: MuderaxConfig, i: int) -> dict:

@@ -83,7 +83,7 @@ def latent_attention(h, w: dict, p: str, m: dict, eps: float):
 
 
 def causal_conv(u, taps, bias):
-    """u [T, C], taps [C, K] (last column = the current token), zeros before the start."""
+    """u [T, C], taps [C, K] ; taps[:, K - 1] weighs the newest input and the history before position 0 is empty."""
     T, K = u.shape[0], taps.shape[1]
     pad = torch.cat([torch.zeros(K - 1, u.shape[1], dtype=u.dtype), u])
     out = bias.expand(T, -1).clone()
@@ -117,7 +117,7 @@ def gated_ffn(h, w: dict, p: str):
 
 
 def moe(h, w: dict, p: str, f: dict):
-    """Top-k of the router's logits, softmax over the chosen logits only, plus the always-on shared expert."""
+    """Top-k of the router's logits, their weights renormalised among themselves by a softmax; the shared expert is added for every row."""
     E, top = int(f["router"]["experts"]), int(f["router"]["top"])
     z = h @ w[p + "router"].T + w[p + "router.b"]
     val, idx = torch.topk(z, top, dim=-1)

@@ -302,7 +302,7 @@ def test_far_key_among_hundreds(device):
 
 @pytest.mark.parametrize("device", DEVICES)
 def test_first_tokens(device):
-    """Positions 0, 1, 2: zeros before the start in the convolution, the recurrence from a zero state, one-key
+    """Positions 0, 1, 2: the convolution's empty history, the recurrence from a zero state, one-key
     attention; as a one-token request, as single tokens from the start, and in a slot that held another sequence."""
     for dtype in modes(device):
         m = Model(HYBRID, device, dtype, max_seqs=1)
@@ -385,6 +385,23 @@ def test_decode_graphs_match_eager():
     graphed = m.run_cut("g", t, [20, 1])
     assert torch.allclose(eager, graphed, atol=1e-5, rtol=1e-5)
     m.check(graphed, m.expect(t), "graph replays")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_borrowed_weights_with_own_constants(device):
+    """A layer that borrows tensors keeps its own window and its own cache; a borrower may come before its lender,
+    and a borrower of a borrower reaches the owner."""
+    a = with_mlp(att(window=5), moe())
+    layers = [shared_of(with_mlp(att(window=17), moe()), 2), rec(), a, shared_of(with_mlp(att(window=3), moe()), 0)]
+    cfgd = config(layers)
+    t = toks(40, seed=40)
+    ref = copy.deepcopy(cfgd)
+    ref["layers"][3]["weights_of"] = 2  # what the chain resolves to
+    for dtype in modes(device):
+        m = Model(cfgd, device, dtype)
+        assert m.cfg.layers[3].weights_of == 2
+        want = oracle.forward(ref, m.weights, t).float()
+        m.check(m.run_cut("b", t, [9, 1]), want, "borrowed weights, own windows")
 
 
 def test_config_round_trip_and_registry(tmp_path):
