@@ -346,6 +346,27 @@ def test_other_sizes(device, name, cfgd):
         m.check(m.run_cut("y", t, [7, 2, 1]), m.expect(t), name + ", portions and decoding")
 
 
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name,cfgd", [
+    ("recurrent first, wide latent, long window",
+     config([with_mlp(rec(width=192, blocks=4, conv=3), moe(8, 3, 64, 128)),
+             with_mlp(att(heads=4, dim=64, rot_dim=64, vdim=32, kv_rank=256, window=100, scale=0.09), moe(8, 3, 64, 128)),
+             att(heads=12, dim=16, rot_dim=32, vdim=16, kv_rank=64, window=33, scale=0.15),
+             shared_of(with_mlp(rec(width=192, blocks=4, conv=3), moe(8, 3, 64, 128)), 0)], width=160, vocab=200)),
+    ("six heads, widths off the MFMA form",
+     config([with_mlp(att(heads=6, dim=24, rot_dim=16, vdim=40, kv_rank=96, window=70, scale=0.16), moe(4, 1, 48, 0)),
+             rec(width=96, blocks=2, conv=2)], width=144, vocab=130)),
+])
+def test_long_prompts_over_many_pages(device, name, cfgd):
+    """Three hundred tokens: windows that span several pages, prompts cut on and off page borders, then decoding."""
+    t = toks(300, vocab=cfgd["vocab"], seed=50)
+    for dtype in modes(device):
+        m = Model(cfgd, device, dtype, max_tokens=320)
+        want = m.expect(t)
+        m.check(m.run_cut("a", t, [280, 1]), want, name + ": prompt, then decoding")
+        m.check(m.run_cut("b", t, [64, 3, 97, 1]), want, name + ": portions")
+
+
 # ---------------------------------------------------------------------------------------------- generation
 @pytest.mark.parametrize("device", DEVICES)
 def test_greedy_generation_through_the_scheduler(device):
