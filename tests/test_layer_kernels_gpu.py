@@ -155,3 +155,35 @@ def test_tiled_dispatch_matches_row_major(gpu, N, K):
             ops.gemm_out(x, wt, b)
             tol = 2e-3 if dt == torch.float32 else 2e-2
             assert torch.allclose(a.float(), b.float(), atol=tol, rtol=tol), (M, dt, float((a.float() - b.float()).abs().max()))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 16, 8), (5, 33, 100), (16, 576, 2048), (17, 96, 96), (70, 130, 257), (300, 512, 384),
+                                    (1113, 160, 256)])
+def test_general_gemm(gpu, dtype, M, N, K):
+    """gemm_rm against the PyTorch reference: every launch shape (skinny split-K, 64 x 64, 128 x 128 tiles), edges in M,
+    N and K, vector and scalar fragment loads, bias, gelu, fp32 and element-type output."""
+    g = torch.Generator().manual_seed(M * N + K)
+    x = torch.randn(M, K, generator=g).to(dtype).to(gpu)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dtype).to(gpu)
+    b = torch.randn(N, generator=g).to(dtype).to(gpu)
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+    for bias, act, odt in ((None, 0, torch.float32), (b, 0, dtype), (b, 1, torch.float32)):
+        out, ref = torch.zeros(M, N, dtype=odt, device=gpu), torch.zeros(M, N, dtype=odt)
+        ops.gemm_rm(x, w, out, bias, act)
+        lref.gemm_rm(x.cpu(), w.cpu(), ref, None if bias is None else bias.cpu(), act)
+        assert torch.allclose(out.cpu().float(), ref.float(), atol=tol, rtol=tol), (bias is not None, act, odt)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_general_gemm_batched_views(gpu, dtype):
+    """Per-head slices of wider buffers as strided views (the query fold and the value up-projection's shapes)."""
+    g = torch.Generator().manual_seed(3)
+    M, H, dn, dr, rk = 37, 5, 24, 8, 40
+    q = torch.randn(M, H, dn + dr, generator=g).to(dtype).to(gpu)
+    w = (torch.randn(H, rk, dn, generator=g) / math.sqrt(dn)).to(dtype).to(gpu)
+    out = torch.zeros(M, H, rk, device=gpu)
+    ops.gemm_rm(q[:, :, :dn].permute(1, 0, 2), w, out.permute(1, 0, 2))
+    ref = torch.einsum("mhd,hrd->mhr", q[:, :, :dn].float().cpu(), w.float().cpu())
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+    assert torch.allclose(out.cpu(), ref, atol=tol, rtol=tol)
