@@ -197,20 +197,30 @@ __global__ __launch_bounds__(256) void latent_flash_kernel(LatentAttnParams p, c
   // stage the 16 query vectors: lane group g fills coordinates g, g + 4, ... (in chunks of 8) of column r
   {
     const float* qa = p.q_abs + (c_row * p.H + (c_ok ? c_head : 0)) * p.rk;
-    for (int d = 8 * g; d < p.rk; d += 32) {
+    for (int d = 8 * g; d < p.rk; d += 32) {  // rk % 32 == 0: the eight floats are two aligned 16-byte loads
+      const f32x4 lo4 = c_ok ? *reinterpret_cast<const f32x4*>(qa + d) : f32x4{0.f, 0.f, 0.f, 0.f};
+      const f32x4 hi4 = c_ok ? *reinterpret_cast<const f32x4*>(qa + d + 4) : f32x4{0.f, 0.f, 0.f, 0.f};
       bf16x8 v;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) v[j] = (bf16)(c_ok ? qa[d + j] : 0.0f);
+      for (int j = 0; j < 4; ++j) v[j] = (bf16)lo4[j], v[4 + j] = (bf16)hi4[j];
       *reinterpret_cast<bf16x8*>(qs + r * ldq + d) = v;
     }
     const bf16* qr = reinterpret_cast<const bf16*>(p.q) + (c_row * p.H + (c_ok ? c_head : 0)) * (p.dn + p.dr) + p.dn;
     const int pp = c_pos < 0 ? 0 : (c_pos >= p.rope_len ? p.rope_len - 1 : c_pos);
     const float2* cs = p.rope + (int64_t)pp * (p.dr / 2);
     for (int d = 8 * g; d < p.dr; d += 32) {
+      // eight rotated coordinates: one 16-byte load when the head's row allows it (dn and dr multiples of 8)
+      bf16x8 raw = zero_bf16x8();
+      if (c_ok) {
+        if (((p.dn + p.dr) % 8 == 0) && (p.dn % 8 == 0)) raw = ld_bf16x8(qr + d);
+        else
+#pragma unroll
+          for (int j = 0; j < 8; ++j) raw[j] = qr[d + j];
+      }
       bf16x8 v;
 #pragma unroll
       for (int j = 0; j < 8; j += 2) {
-        const float a = c_ok ? (float)qr[d + j] : 0.0f, b = c_ok ? (float)qr[d + j + 1] : 0.0f;
+        const float a = (float)raw[j], b = (float)raw[j + 1];
         const float2 t = cs[(d + j) / 2];
         v[j] = (bf16)(a * t.x - b * t.y);
         v[j + 1] = (bf16)(b * t.x + a * t.y);
