@@ -34,6 +34,16 @@ DEV f32x4 mfma16x16x32(const bf16x8& a, const bf16x8& b, const f32x4& c) {
 
 DEV bf16x8 ld_bf16x8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
+// Loads through a pointer KNOWN to be global memory.  A pointer that reaches a kernel inside a by-value parameter
+// struct is a generic (flat) pointer to the compiler; flat loads count on both memory counters and cannot overlap
+// with LDS traffic the way global loads do.  Casting to the global address space where the kernel knows better turns
+// them into global_load instructions.
+#define DSSE_GLOBAL __attribute__((address_space(1)))
+template <typename V>
+DEV V ld_global(const void* p) {
+  return *(const DSSE_GLOBAL V*)(p);
+}
+
 DEV bf16x8 zero_bf16x8() {
   bf16x8 z;
 #pragma unroll

@@ -25,7 +25,7 @@ DEV typename Frag<T>::V load_frag(const T* row, int k, int K, bool valid, bool v
 #pragma unroll
   for (int j = 0; j < F::PER; ++j) v[j] = (T)0.0f;
   if (!valid || k >= K) return v;
-  if (vec && k + F::PER <= K) return *reinterpret_cast<const typename F::V*>(row + k);
+  if (vec && k + F::PER <= K) return ld_global<typename F::V>(row + k);
 #pragma unroll
   for (int j = 0; j < F::PER; ++j)
     if (k + j < K) v[j] = row[k + j];

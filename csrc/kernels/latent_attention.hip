@@ -259,7 +259,7 @@ __global__ __launch_bounds__(256) void latent_flash_kernel(LatentAttnParams p, c
     const bf16* vrow = vt + ((int64_t)blk * p.rk + r) * kBS + 8 * g;  // dim r of value tile 0, positions 8g..8g+7
     bf16x8 vf[NT];
 #pragma unroll
-    for (int n = 0; n < NT; ++n) vf[n] = ld_bf16x8(vrow + (int64_t)n * 16 * kBS);
+    for (int n = 0; n < NT; ++n) vf[n] = ld_global<bf16x8>(vrow + (int64_t)n * 16 * kBS);
     f32x4 s0 = f32x4{0.f, 0.f, 0.f, 0.f}, s1 = s0;
     // six k-steps at a time: their twelve key loads are issued before the first MFMA needs one (a single wave per
     // work item has nothing else to hide the load latency behind)
@@ -268,8 +268,8 @@ __global__ __launch_bounds__(256) void latent_flash_kernel(LatentAttnParams p, c
 #pragma unroll
       for (int u = 0; u < 6; ++u) {
         const int s = sb + u < nks ? sb + u : nks - 1;  // past the end: a valid address, the product is skipped
-        ka[u] = ld_bf16x8(krow0 + 32 * s);
-        kb[u] = ld_bf16x8(krow1 + 32 * s);
+        ka[u] = ld_global<bf16x8>(krow0 + 32 * s);
+        kb[u] = ld_global<bf16x8>(krow1 + 32 * s);
         qb[u] = *reinterpret_cast<const bf16x8*>(qs + r * ldq + 32 * s + 8 * g);
       }
 #pragma unroll
