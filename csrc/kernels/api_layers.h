@@ -103,6 +103,8 @@ struct LruScanParams {
   void* out;             // [T, C] element type: state * y
   int nseq, C, bw, rows; // rows = T
   int coeff;             // 1: compute (a, b) for all rows first; 0: gates already hold them (a later sequence group)
+  float* chunk_a;        // [rows / 32 + nseq + 1, C] scratch of the chunked walk (prompt portions), or null
+  float* chunk_b;
   float c;               // 8: log a = -c r softplus(lam)
   int f32;
 };

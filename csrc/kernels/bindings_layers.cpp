@@ -288,7 +288,7 @@ void conv_state(const Tensor& in, const Tensor& taps, const OptTensor& bias, Ten
 
 void lru_scan(const Tensor& u, Tensor& gates, const Tensor& y, const Tensor& lam, Tensor& state,
               const Tensor& q_start, const Tensor& q_len, const Tensor& ctx_len, const Tensor& state_slot, Tensor& out,
-              double c, const OptTensor& y_bias, bool coeff) {
+              double c, const OptTensor& y_bias, bool coeff, const OptTensor& scratch) {
   f32t(u, "u");
   f32t(gates, "gates");
   f32t(y, "y");
@@ -314,6 +314,15 @@ void lru_scan(const Tensor& u, Tensor& gates, const Tensor& y, const Tensor& lam
   }
   p.rows = (int)u.size(0);
   p.coeff = coeff ? 1 : 0;
+  if (scratch.has_value()) {  // [2, slots, C] with slots >= rows / 32 + sequences + 1: the chunked walk's scratch
+    f32t(*scratch, "scratch");
+    const int64_t slots = p.rows / 32 + p.nseq + 1;
+    TORCH_CHECK(scratch->dim() == 3 && scratch->size(0) == 2 && scratch->size(1) >= slots && scratch->size(2) == C,
+                "lru_scan scratch must be [2, >= rows / 32 + sequences + 1, C]");
+    p.chunk_a = scratch->data_ptr<float>();
+    p.chunk_b = p.chunk_a + scratch->size(1) * (int64_t)C;
+    TORCH_CHECK((p.rows + 31) / 32 <= 65535, "lru_scan: too many rows");
+  }
   p.lam = lam.data_ptr();
   p.state = state.data_ptr<float>();
   p.q_start = q_start.data_ptr<int>();
@@ -498,7 +507,8 @@ TORCH_LIBRARY_FRAGMENT(dsse, m) {
   m.def("conv_state(Tensor inp, Tensor taps, Tensor? bias, Tensor(a!) tail, Tensor q_start, Tensor q_len, "
         "Tensor ctx_len, Tensor state_slot, Tensor(b!) out, Tensor(c!) out_b, Tensor? in_bias=None) -> ()");
   m.def("lru_scan(Tensor u, Tensor(c!) gates, Tensor y, Tensor lam, Tensor(a!) state, Tensor q_start, Tensor q_len, "
-        "Tensor ctx_len, Tensor state_slot, Tensor(b!) out, float c, Tensor? y_bias=None, bool coeff=True) -> ()");
+        "Tensor ctx_len, Tensor state_slot, Tensor(b!) out, float c, Tensor? y_bias=None, bool coeff=True, "
+        "Tensor(d!)? scratch=None) -> ()");
   m.def("moe_router(Tensor x, Tensor w, Tensor? b, Tensor(a!) topk_idx, Tensor(b!) topk_w) -> ()");
   m.def("moe_topk(Tensor logits, Tensor(a!) topk_idx, Tensor(b!) topk_w) -> ()");
   m.def("moe_ffn(Tensor x, Tensor topk_idx, Tensor topk_w, Tensor gate, Tensor up, Tensor down, Tensor? sgate, "

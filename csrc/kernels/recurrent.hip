@@ -125,6 +125,71 @@ __global__ __launch_bounds__(256) void lru_scan_kernel(LruScanParams p) {
   *st = S;
 }
 
+// Prompt portions: the walk in three phases so that no thread takes more than ~3 x 32 dependent steps.  A chunk is
+// kScanRows rows of one sequence; its scratch slot is (first row) / kScanRows + (sequence index), which is unique because
+// sequences are packed in row order.
+//   1. per chunk, in parallel: A = prod a_t and B = the chunk's walk from S = 0          (S_end = A S_in + B)
+//   2. per sequence: the chunks in order -- each chunk's incoming state replaces its B, the last one is the slot's state
+//   3. per chunk, in parallel: the walk from the incoming state, times gelu(branch + bias)
+constexpr int kScanRows = 32;
+constexpr int kChunkedFrom = 128;  // rows of a step from which the walk is chunked (below: one thread per sequence)
+
+DEV int scan_slot(int row0, int t0, int seq) { return (row0 + t0) / kScanRows + seq; }
+
+__global__ __launch_bounds__(256) void lru_chunk_reduce_kernel(LruScanParams p) {
+  const int seq = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int ql = p.q_len[seq], t0 = blockIdx.z * kScanRows;
+  if (c >= p.C || t0 >= ql) return;
+  const int t1 = t0 + kScanRows < ql ? t0 + kScanRows : ql;
+  const int row0 = p.q_start[seq];
+  const int b = c / p.bw, o = c % p.bw;
+  const float* ab = p.gates + (int64_t)row0 * 2 * p.C + (int64_t)b * 2 * p.bw + o;
+  float A = 1.0f, B = 0.0f;
+  for (int t = t0; t < t1; ++t) {
+    const float a = ab[(int64_t)t * 2 * p.C];
+    B = a * B + ab[(int64_t)t * 2 * p.C + p.bw];
+    A *= a;
+  }
+  const int64_t s = (int64_t)scan_slot(row0, t0, seq) * p.C + c;
+  p.chunk_a[s] = A;
+  p.chunk_b[s] = B;
+}
+
+__global__ __launch_bounds__(256) void lru_chunk_carry_kernel(LruScanParams p) {
+  const int seq = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int ql = p.q_len[seq];
+  if (c >= p.C || ql <= 0) return;
+  const int row0 = p.q_start[seq];
+  float* st = p.state + (int64_t)p.state_slot[seq] * p.C + c;
+  float S = p.ctx_len[seq] - ql == 0 ? 0.0f : *st;
+  for (int t0 = 0; t0 < ql; t0 += kScanRows) {
+    const int64_t s = (int64_t)scan_slot(row0, t0, seq) * p.C + c;
+    const float next = p.chunk_a[s] * S + p.chunk_b[s];
+    p.chunk_b[s] = S;  // the chunk's incoming state
+    S = next;
+  }
+  *st = S;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void lru_chunk_apply_kernel(LruScanParams p) {
+  const int seq = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int ql = p.q_len[seq], t0 = blockIdx.z * kScanRows;
+  if (c >= p.C || t0 >= ql) return;
+  const int t1 = t0 + kScanRows < ql ? t0 + kScanRows : ql;
+  const int row0 = p.q_start[seq];
+  const int b = c / p.bw, o = c % p.bw;
+  const float yb = p.y_bias ? (float)reinterpret_cast<const T*>(p.y_bias)[c] : 0.0f;
+  const float* ab = p.gates + (int64_t)row0 * 2 * p.C + (int64_t)b * 2 * p.bw + o;
+  const float* y = p.y + (int64_t)row0 * p.C + c;
+  T* out = reinterpret_cast<T*>(p.out) + (int64_t)row0 * p.C + c;
+  float S = p.chunk_b[(int64_t)scan_slot(row0, t0, seq) * p.C + c];
+  for (int t = t0; t < t1; ++t) {
+    S = ab[(int64_t)t * 2 * p.C] * S + ab[(int64_t)t * 2 * p.C + p.bw];
+    out[(int64_t)t * p.C] = (T)(S * gelu_tanh_f(y[(int64_t)t * p.C] + yb));
+  }
+}
+
 }  // namespace
 }  // namespace dsse
 
@@ -146,12 +211,19 @@ extern "C" hipError_t dsse_lru_scan(const dsse::LruScanParams* p, hipStream_t st
   if (p->nseq <= 0 || p->rows <= 0) return hipSuccess;
   dim3 cgrid(p->rows, (p->C + 255) / 256);
   dim3 grid((p->C + 255) / 256, p->nseq);
-  if (p->f32) {
-    if (p->coeff) hipLaunchKernelGGL(dsse::lru_coeff_kernel<float>, cgrid, dim3(256), 0, st, *p, p->rows);
-    hipLaunchKernelGGL(dsse::lru_scan_kernel<float>, grid, dim3(256), 0, st, *p);
-  } else {
-    if (p->coeff) hipLaunchKernelGGL(dsse::lru_coeff_kernel<bf16>, cgrid, dim3(256), 0, st, *p, p->rows);
-    hipLaunchKernelGGL(dsse::lru_scan_kernel<bf16>, grid, dim3(256), 0, st, *p);
+  if (p->coeff) {
+    if (p->f32) hipLaunchKernelGGL(dsse::lru_coeff_kernel<float>, cgrid, dim3(256), 0, st, *p, p->rows);
+    else hipLaunchKernelGGL(dsse::lru_coeff_kernel<bf16>, cgrid, dim3(256), 0, st, *p, p->rows);
   }
+  if (p->chunk_a && p->chunk_b && p->rows >= dsse::kChunkedFrom) {  // prompt portions: the three-phase walk
+    dim3 zgrid((p->C + 255) / 256, p->nseq, (p->rows + dsse::kScanRows - 1) / dsse::kScanRows);
+    hipLaunchKernelGGL(dsse::lru_chunk_reduce_kernel, zgrid, dim3(256), 0, st, *p);
+    hipLaunchKernelGGL(dsse::lru_chunk_carry_kernel, grid, dim3(256), 0, st, *p);
+    if (p->f32) hipLaunchKernelGGL(dsse::lru_chunk_apply_kernel<float>, zgrid, dim3(256), 0, st, *p);
+    else hipLaunchKernelGGL(dsse::lru_chunk_apply_kernel<bf16>, zgrid, dim3(256), 0, st, *p);
+    return hipGetLastError();
+  }
+  if (p->f32) hipLaunchKernelGGL(dsse::lru_scan_kernel<float>, grid, dim3(256), 0, st, *p);
+  else hipLaunchKernelGGL(dsse::lru_scan_kernel<bf16>, grid, dim3(256), 0, st, *p);
   return hipGetLastError();
 }

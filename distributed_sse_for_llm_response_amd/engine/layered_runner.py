@@ -96,6 +96,8 @@ class LayeredRunner(RunnerBase):
             d["ub"], d["hs"] = (torch.zeros(M * C, **el) for _ in range(2))
             d["yr"], d["ux"], d["u"] = (torch.zeros(M * C, **f32) for _ in range(3))
             d["gates"] = torch.zeros(M * 2 * C, **f32)
+            # chunked walk of the recurrence over prompt portions: (A, B) per 32-row chunk
+            d["scan"] = torch.zeros(2 * (M // 32 + max(M, self.max_batch) + 2) * C, **f32) if M >= 128 else None
         if moe:
             top = max(f.top for f in moe)
             d["tki"] = torch.zeros(M * top, device=dev, dtype=torch.int32)
@@ -175,8 +177,12 @@ class LayeredRunner(RunnerBase):
                            Lw.x_b)
         ops.gemm_rm(ub.view(M, nb, bw).permute(1, 0, 2), Lw.gates, gates.permute(1, 0, 2), bias=Lw.gates_b)
         for i, g in enumerate(groups):
+            scr = d.get("scan")
+            if scr is not None:
+                slots = M // 32 + g["ql"].numel() + 1
+                scr = scr[:2 * slots * C].view(2, slots, C)
             ops.lru_scan(u, gates, yr, Lw.lam, self.state.state[li], g["qs"], g["ql"], g["ctx"], g["ss"], hs,
-                         LRU_DECAY_SCALE, Lw.y_b, i == 0)
+                         LRU_DECAY_SCALE, Lw.y_b, i == 0, scr)
         self._lin(hs, Lw.o, Lw.o_t, d["y"])
 
     def _moe(self, f, Fw, M: int, d: dict):

@@ -89,12 +89,14 @@ def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, 
 
 
 def lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, c: float, y_bias=None,
-             coeff: bool = True):
+             coeff: bool = True, scratch=None):
     """Real-gated linear recurrence continued from each sequence's slot state; out = state · gelu(y + y_bias).
     coeff: turn the gate pre-activations of ALL rows into the recurrence's coefficients first (in place); pass False
-    for a further sequence group of the same step."""
+    for a further sequence group of the same step.  scratch (fp32 [2, rows / 32 + sequences + 1, C]): steps of 128 rows
+    or more walk in three phases over 32-row chunks instead of one thread per sequence and channel."""
     if _hip(u):
-        torch.ops.dsse.lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, c, y_bias, coeff)
+        torch.ops.dsse.lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, c, y_bias, coeff,
+                                scratch)
     else:
         lref.lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, c, y_bias, coeff)
 
