@@ -151,6 +151,7 @@ struct MoeGroupedParams {
   float* o;              // [M * S, W]
   int M, W, F, Fs, E, top, S, ldh, max_tiles;
   int vec_w, vec_h;      // 16-byte fragment loads allowed on rows W wide / on rows of h
+  int lds_tiles;         // 1: enough rows for the LDS-staged tiles (prompt portions); 0: the register-direct kernels
   int f32;
 };
 

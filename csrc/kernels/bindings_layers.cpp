@@ -475,6 +475,7 @@ void moe_grouped(const Tensor& x, const Tensor& topk_idx, const Tensor& topk_w, 
   const int per = p.f32 ? 4 : 8;
   p.vec_w = p.W % per == 0;
   p.vec_h = p.ldh % per == 0 && p.F % per == 0;
+  p.lds_tiles = ids >= 256;  // prompt-sized: most 64-row tiles are full
   DSSE_CHECK_HIP(dsse_moe_grouped(&p, cur_stream()));
 }
 

@@ -317,6 +317,134 @@ __global__ __launch_bounds__(256) void moe_down_kernel(MoeGroupedParams p) {
   }
 }
 
+// Prompt-sized row counts (bf16, widths multiples of 8): the same two GEMMs with both operands staged through LDS.
+// A workgroup owns a 64-row tile of one expert times 128 weight rows (MODE 0: 64 hidden units' gate rows and the same
+// units' up rows; MODE 1: 128 output columns of the down projection) and walks K in chunks of 64: 256 threads copy the
+// next chunk global -> registers while the MFMAs read the current one from LDS (two buffers, rows padded to 144 bytes so
+// that a fragment read touches every bank once).  Each wave holds 4 row tiles x 2 weight tiles of accumulators: 8 MFMAs
+// per 6 fragment reads from LDS, and every weight element leaves global memory once per 64 rows instead of once per
+// wave.
+constexpr int kLdsK = 64;            // K elements per chunk
+constexpr int kLdsRow = kLdsK + 8;   // padded LDS row, bf16 elements
+
+template <int MODE>
+__global__ __launch_bounds__(256) void moe_tile_lds_kernel(MoeGroupedParams p) {
+  __shared__ __align__(16) bf16 sa[2][64 * kLdsRow];
+  __shared__ __align__(16) bf16 sb[2][128 * kLdsRow];
+  const int t = blockIdx.y;
+  if (t >= *p.num_tiles) return;
+  const int e = p.tile_expert[t];
+  const bool sh = e >= p.E;
+  const int Fe = sh ? p.Fs : p.F;
+  const int K = MODE == 0 ? p.W : Fe;          // reduction length
+  const int N = MODE == 0 ? Fe : p.W;          // weight rows of one kind
+  const int n0 = blockIdx.x * (MODE == 0 ? 64 : 128);
+  if (n0 >= N) return;
+  const int* ids = p.sorted + t * kMoeRows;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
+  const bf16* X = reinterpret_cast<const bf16*>(MODE == 0 ? p.x : p.h);
+  const int ldx = MODE == 0 ? p.W : p.ldh;
+  const bf16 *w0, *w1;  // MODE 0: gate, up; MODE 1: down (w1 unused)
+  if (MODE == 0) {
+    w0 = sh ? reinterpret_cast<const bf16*>(p.sgate) : reinterpret_cast<const bf16*>(p.gate) + (int64_t)e * p.F * p.W;
+    w1 = sh ? reinterpret_cast<const bf16*>(p.sup) : reinterpret_cast<const bf16*>(p.up) + (int64_t)e * p.F * p.W;
+  } else {
+    w0 = sh ? reinterpret_cast<const bf16*>(p.sdown) : reinterpret_cast<const bf16*>(p.down) + (int64_t)e * p.W * p.F;
+    w1 = w0;
+  }
+  // this thread's copies per chunk: 2 of the A tile (64 rows x 8 sixteen-byte pieces), 4 of the B tile (128 rows x 8)
+  const bf16* ap[2];
+  const bf16* bp[4];
+  int ak[2], bk[4], ao[2], bo[4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int idx = tid + 256 * i, row = idx >> 3, pc = idx & 7;
+    const int id = ids[row];
+    ap[i] = id >= 0 ? X + (int64_t)(MODE == 0 ? id / p.S : id) * ldx : nullptr;
+    ak[i] = 8 * pc;
+    ao[i] = row * kLdsRow + 8 * pc;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int idx = tid + 256 * i, row = idx >> 3, pc = idx & 7;
+    int n;
+    const bf16* base;
+    if (MODE == 0) {
+      n = n0 + (row & 63);
+      base = row < 64 ? w0 : w1;
+    } else {
+      n = n0 + row;
+      base = w0;
+    }
+    bp[i] = n < N ? base + (int64_t)n * K : nullptr;
+    bk[i] = 8 * pc;
+    bo[i] = row * kLdsRow + 8 * pc;
+  }
+  bf16x8 ra[2], rb[4];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      ra[i] = (ap[i] && k0 + ak[i] < K) ? ld_global<bf16x8>(ap[i] + k0 + ak[i]) : zero_bf16x8();
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      rb[i] = (bp[i] && k0 + bk[i] < K) ? ld_global<bf16x8>(bp[i] + k0 + bk[i]) : zero_bf16x8();
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) *reinterpret_cast<bf16x8*>(&sa[buf][ao[i]]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(&sb[buf][bo[i]]) = rb[i];
+  };
+  f32x4 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc[i][0] = acc[i][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // this wave's two weight tiles inside the B tile
+  const int br0 = MODE == 0 ? 16 * wave : 32 * wave;
+  const int br1 = MODE == 0 ? 64 + 16 * wave : 32 * wave + 16;
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  const int nchunks = (K + kLdsK - 1) / kLdsK;
+  for (int c = 0; c < nchunks; ++c) {
+    const int buf = c & 1;
+    if (c + 1 < nchunks) fetch((c + 1) * kLdsK);
+#pragma unroll
+    for (int ks = 0; ks < kLdsK; ks += 32) {
+      const bf16x8 b0 = *reinterpret_cast<const bf16x8*>(&sb[buf][(br0 + r) * kLdsRow + ks + 8 * g]);
+      const bf16x8 b1 = *reinterpret_cast<const bf16x8*>(&sb[buf][(br1 + r) * kLdsRow + ks + 8 * g]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(&sa[buf][(16 * i + r) * kLdsRow + ks + 8 * g]);
+        acc[i][0] = mfma16x16x32(a, b0, acc[i][0]);
+        acc[i][1] = mfma16x16x32(a, b1, acc[i][1]);
+      }
+    }
+    if (c + 1 < nchunks) stash(buf ^ 1);  // the other buffer: its readers finished before the previous barrier
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int id = ids[16 * i + 4 * g + j];
+      if (id < 0) continue;
+      if (MODE == 0) {
+        const int f = n0 + 16 * wave + r;
+        if (f >= N) continue;
+        const float gv = acc[i][0][j];
+        reinterpret_cast<bf16*>(p.h)[(int64_t)id * p.ldh + f] = (bf16)(gv / (1.0f + expf(-gv)) * acc[i][1][j]);
+      } else {
+        const int row = id / p.S, k = id % p.S;
+        const float wgt = k < p.top ? p.topk_w[row * p.top + k] : 1.0f;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const int d = n0 + 32 * wave + 16 * q + r;
+          if (d < N) p.o[(int64_t)id * p.W + d] = wgt * acc[i][q][j];
+        }
+      }
+    }
+}
+
 }  // namespace
 }  // namespace dsse
 
@@ -344,6 +472,13 @@ extern "C" hipError_t dsse_moe_grouped(const dsse::MoeGroupedParams* p, hipStrea
   hipLaunchKernelGGL(dsse::moe_align_kernel, dim3(1), dim3(256), sizeof(int) * (3 * NE + 1), st, *p);
   const int fmax = p->F > p->Fs ? p->F : p->Fs;
   dim3 g1((fmax + 15) / 16, p->max_tiles), g2((p->W + 15) / 16, p->max_tiles);
+  // prompt-sized steps in bf16 with 16-byte-aligned rows: operands staged through LDS
+  if (!p->f32 && p->lds_tiles && p->W % 8 == 0 && p->F % 8 == 0 && p->Fs % 8 == 0 && p->ldh % 8 == 0) {
+    dim3 l1((fmax + 63) / 64, p->max_tiles), l2((p->W + 127) / 128, p->max_tiles);
+    hipLaunchKernelGGL(dsse::moe_tile_lds_kernel<0>, l1, dim3(256), 0, st, *p);
+    hipLaunchKernelGGL(dsse::moe_tile_lds_kernel<1>, l2, dim3(256), 0, st, *p);
+    return hipGetLastError();
+  }
   if (p->f32) {
     hipLaunchKernelGGL(dsse::moe_gate_up_kernel<float>, g1, dim3(256), 0, st, *p);
     hipLaunchKernelGGL(dsse::moe_down_kernel<float>, g2, dim3(256), 0, st, *p);
