@@ -100,3 +100,31 @@ class RecurrentStateCache:
         for group in (self.state, self.tail):
             for t in group.values():
                 t.index_copy_(0, dst_idx, t.index_select(0, src_idx))
+
+
+class PagedKVCache:
+    """Paged keys and values of softmax-attention layers with any head widths: per attention run one key tensor
+    [blocks, PAGE, G, D] and one value tensor [blocks, PAGE, G, V] in the engine's element type, indexed with the same
+    block tables and allocator as the other caches (a page id means the same page in every run).  ``shapes`` maps a
+    run's key -> (G, D, V); a layer that runs several times (a looped span) has one entry per run."""
+
+    def __init__(self, shapes: dict, num_blocks: int, device, dtype=torch.bfloat16):
+        self.num_blocks = num_blocks
+        self.k = {r: torch.zeros(num_blocks, PAGE, g, d, device=device, dtype=dtype) for r, (g, d, _) in shapes.items()}
+        self.v = {r: torch.zeros(num_blocks, PAGE, g, v, device=device, dtype=dtype) for r, (g, _, v) in shapes.items()}
+
+    @staticmethod
+    def bytes_per_block(shapes: dict, elem_bytes: int = 2) -> int:
+        return max(1, sum(g * (d + v) for g, d, v in shapes.values()) * PAGE * elem_bytes)
+
+
+class MatrixStateCache(RecurrentStateCache):
+    """Per-sequence state of matrix-state mixers, indexed by the decode slot like RecurrentStateCache: per run the
+    fp32 state [slots, H, D, V] and, for mixers with a short convolution in front, its tail [slots, taps - 1, C].
+    ``shapes`` maps a run's key -> ((H, D, V), C, taps) with C = 0 for mixers without a convolution."""
+
+    def __init__(self, shapes: dict, num_slots: int, device):
+        self.num_slots = num_slots
+        self.state = {r: torch.zeros(num_slots, *s, device=device, dtype=torch.float32) for r, (s, _, _) in shapes.items()}
+        self.tail = {r: torch.zeros(num_slots, k - 1, c, device=device, dtype=torch.float32)
+                     for r, (_, c, k) in shapes.items() if c > 0 and k > 1}

@@ -31,8 +31,9 @@ import torch
 
 from .. import ops
 from ..models.muderax import LRU_DECAY_SCALE
+from ..models.surodra import UNIT_EPS
 from ..parallel.comm import TPComm
-from .kv_cache import PAGE, LatentKVCache, RecurrentStateCache
+from .kv_cache import PAGE, LatentKVCache, MatrixStateCache, PagedKVCache, RecurrentStateCache
 from .model_runner import RunnerBase, _capture, batch_buckets
 from .weights import LayeredWeights
 
@@ -58,10 +59,20 @@ class LayeredRunner(RunnerBase):
         self.use_graphs = (self.device.type == "cuda") if use_graphs is None else use_graphs
         cfg, dev = self.cfg, self.device
         self._init_slots(max_batch, self.max_blocks, cfg.vocab_size, dev, self.comm)
+        self.num_blocks = num_blocks
+        self.prenorm = getattr(cfg, "family", "") == "surodra"   # pre-norm blocks with matrix-state mixers
+        if self.prenorm:
+            self._setup_prenorm()
+        else:
+            self._setup_sandwich()
+        self._dec = self._buffers(max_batch)  # static decode activations (captured graphs read and write them)
+
+    def _setup_sandwich(self) -> None:
+        cfg, dev, max_batch = self.cfg, self.device, self.max_batch
         att = {i: L.mixer for i, L in enumerate(cfg.layers) if L.kind == "latent_attention"}
         rec = {i: L.mixer for i, L in enumerate(cfg.layers) if L.kind == "rglru"}
         flash = {i: m.kv_rank for i, m in att.items() if ops.latent_flash_ok(self.dtype, m.kv_rank, m.rot_dim)}
-        self.kv = LatentKVCache({i: m.kv_rank + m.rot_dim for i, m in att.items()}, num_blocks, dev, self.dtype,
+        self.kv = LatentKVCache({i: m.kv_rank + m.rot_dim for i, m in att.items()}, self.num_blocks, dev, self.dtype,
                                 transposed=flash)
         self.state = RecurrentStateCache({i: (m.width, m.conv) for i, m in rec.items()}, max_batch, dev)
         # one rotation table per distinct (rotation, rotated width)
@@ -69,11 +80,31 @@ class LayeredRunner(RunnerBase):
         for m in att.values():
             key = (m.rot, m.rot_dim)
             if key not in self._rope:
-                self._rope[key] = m.rot.table(max_model_len + 1, m.rot_dim, dev)
-        self._dec = self._buffers(max_batch)  # static decode activations (captured graphs read and write them)
+                self._rope[key] = m.rot.table(self.max_model_len + 1, m.rot_dim, dev)
         words = max((ops.latent_flash_part_floats(max_batch, m.heads, 16, 16, m.kv_rank) for i, m in att.items()
                      if i in flash), default=0)
         self._flash_part = torch.zeros(max(1, words), device=dev, dtype=torch.float32)
+
+    def _setup_prenorm(self) -> None:
+        """Caches and state of a pre-norm design, keyed by layer RUN: a layer inside a looped span runs several times
+        with the same weights and has its own pages and state slots each time."""
+        cfg, dev = self.cfg, self.device
+        self.runs = cfg.runs()
+        kv, st, self._rope = {}, {}, {}
+        for r in self.runs:
+            L, m = cfg.layers[r.layer], cfg.layers[r.layer].mixer
+            if L.kind == "delta":
+                st[r.index] = ((m.heads, m.dim, m.vdim), 2 * m.kv_heads * m.dim + m.heads * m.vdim, m.conv)
+            elif L.kind == "parallel":
+                kv[r.index] = (m.left.kv_heads, m.left.dim, m.left.vdim)
+                st[r.index] = ((m.right.heads, m.right.dim, m.right.vdim), 0, 1)
+            else:
+                st[r.index] = ((m.heads, m.dim, m.vdim), 0, 1)
+            rot = m.left.rot if L.kind == "parallel" else getattr(m, "rot", None)
+            if rot is not None and rot.dims > 0 and rot not in self._rope:
+                self._rope[rot] = rot.table(self.max_model_len + 1, dev)
+        self.kv = PagedKVCache(kv, self.num_blocks, dev, self.dtype)
+        self.state = MatrixStateCache(st, self.max_batch, dev)
 
     # ------------------------------------------------------------------ buffers
     def _buffers(self, M: int) -> dict:
@@ -82,6 +113,9 @@ class LayeredRunner(RunnerBase):
         el = dict(device=dev, dtype=self.dtype)
         W = cfg.width
         d = {"resid": torch.zeros(M, W, **f32), "xb": torch.zeros(M, W, **el), "y": torch.zeros(M, W, **f32)}
+        if self.prenorm:
+            d.update(self._prenorm_buffers(M))
+            return d
         att = [L.mixer for L in cfg.layers if L.kind == "latent_attention"]
         rec = [L.mixer for L in cfg.layers if L.kind == "rglru"]
         moe = [L.mlp for L in cfg.layers if L.mlp is not None]
@@ -204,6 +238,9 @@ class LayeredRunner(RunnerBase):
         attention work items ws / wt of qt rows).  trace (a list) receives a copy of the stream after every layer."""
         cfg, eps = self.cfg, self.cfg.eps
         ops.embed_rows(ids, self.w.embed, d["resid"], d["xb"])
+        if self.prenorm:
+            self._prenorm_layers(M, d, ids, pos, slots, groups, trace)
+            return
         for li, (L, Lw) in enumerate(zip(cfg.layers, self.w.layers)):
             if L.kind == "latent_attention":
                 self._attention(li, L.mixer, Lw.mix, M, d, pos, slots, groups)
@@ -217,10 +254,164 @@ class LayeredRunner(RunnerBase):
                 trace.append(d["resid"].clone())
 
     def _lm_head(self, rows, logits) -> None:
-        """rows: fp32 stream rows (not normed yet) -> final one-number norm -> head GEMM."""
+        """rows: fp32 stream rows (not normed yet) -> final norm -> head GEMM (-> logit scale and cap)."""
+        rows = rows.contiguous()
         xn = torch.empty(rows.shape, device=rows.device, dtype=self.dtype)
-        ops.scalar_norm(None, self.w.final_norm, rows.contiguous(), xn, self.cfg.eps)
-        self._lin(xn, self.w.head, self.w.head_t, logits)
+        self._head(rows, xn, logits)
+
+    def _head(self, resid, xn, logits) -> None:
+        if self.prenorm:
+            n, cfg = self.w.final_norm, self.cfg
+            ops.stream_step(None, 0.0, resid, None, None, None, n.alpha, n.w, n.b, xn)
+            self._lin(xn, self.w.head, self.w.head_t, logits)
+            if cfg.logit_scale != 1.0 or cfg.logit_softcap > 0:
+                ops.logit_cap(logits, cfg.logit_scale, cfg.logit_softcap)
+        else:
+            ops.scalar_norm(None, self.w.final_norm, resid, xn, self.cfg.eps)
+            self._lin(xn, self.w.head, self.w.head_t, logits)
+
+    # ------------------------------------------------------------------ pre-norm designs, matrix-state mixers
+    def _prenorm_buffers(self, M: int) -> dict:
+        """Scratch of a step of M rows, each sized for the widest layer: `big` / `small` take the fused projections'
+        fp32 outputs (their column ranges are the mixer's q, k, v, gates), `cv` the convolution's, `z` the per-channel
+        decays, `qa` the attention's normed and rotated queries, `o` the recurrences' outputs, `ao` a mixer's gated
+        output in the element type (the output projection's input), `y2` the second mixer of a parallel pair."""
+        cfg, dev = self.cfg, self.device
+        f32 = dict(device=dev, dtype=torch.float32)
+        el = dict(device=dev, dtype=self.dtype)
+        big = small = cv = z = qa = o = ff = 1
+        for i, L in enumerate(cfg.layers):
+            m = L.mixer
+            if L.kind == "delta":
+                c = 2 * m.kv_heads * m.dim + m.heads * m.vdim
+                big, small, cv, o = max(big, c + m.heads * m.vdim), max(small, 2 * m.heads), max(cv, c), max(o, m.heads * m.vdim)
+            elif L.kind == "parallel":
+                a, r = m.left, m.right
+                nl = (a.heads + a.kv_heads) * a.dim + a.kv_heads * a.vdim
+                big = max(big, nl + 2 * r.heads * (r.dim + r.vdim))
+                small = max(small, a.heads + self.w.layers[i].mix.a2.shape[1])
+                z, qa = max(z, r.heads * r.dim), max(qa, a.heads * a.dim)
+                o = max(o, a.heads * a.vdim, r.heads * r.vdim)
+            else:
+                big, o = max(big, 2 * m.heads * (m.dim + m.vdim)), max(o, m.heads * m.vdim)
+            if L.mlp is not None:
+                ff = max(ff, L.mlp.ff)
+        return {"y2": torch.zeros(M, cfg.width, **f32), "big": torch.zeros(M * big, **f32),
+                "small": torch.zeros(M * small, **f32), "cv": torch.zeros(M * cv, **f32), "z": torch.zeros(M * z, **f32),
+                "qa": torch.zeros(M * qa, **f32), "o": torch.zeros(M * o, **f32), "ao": torch.zeros(M * o, **el),
+                "gu": torch.zeros(M * 2 * ff, **f32), "h": torch.zeros(M * ff, **el)}
+
+    def _prenorm_layers(self, M: int, d: dict, ids, pos, slots, groups: list, trace: list | None) -> None:
+        """Every layer run over M packed rows.  Between sublayers ONE stream_step adds the finished sublayer's output
+        (times the residual multiplier), what a new pass of the looped span adds (the embedding again, the pass's
+        vector) and applies the next sublayer's norm; the last output is added before the head's norm."""
+        cfg, w = self.cfg, self.w
+        mult = cfg.residual_mult
+        pending = None
+        for run in self.runs:
+            L, Lw = cfg.layers[run.layer], w.layers[run.layer]
+            t = run.pass_no
+            n = Lw.norm1
+            ops.stream_step(pending, mult, d["resid"], ids if t > 0 else None, w.embed if t > 0 else None,
+                            w.step[t] if t >= 0 else None, n.alpha, n.w, n.b, d["xb"])
+            getattr(self, "_" + L.kind)(run.index, L.mixer, Lw.mix, M, d, pos, slots, groups)
+            if L.mlp is not None:
+                n = Lw.norm2
+                ops.stream_step(d["y"], mult, d["resid"], None, None, None, n.alpha, n.w, n.b, d["xb"])
+                self._dense_ff(L.mlp, Lw.mlp, M, d)
+            pending = d["y"]
+            if trace is not None:
+                ops.stream_step(pending, mult, d["resid"], None, None, None, None, None, None, None)
+                pending = None
+                trace.append(d["resid"].clone())
+        if pending is not None:
+            ops.stream_step(pending, mult, d["resid"], None, None, None, None, None, None, None)
+
+    def _dense_ff(self, f, Fw, M: int, d: dict) -> None:
+        gu = d["gu"][:M * 2 * f.ff].view(M, 2 * f.ff)
+        h = d["h"][:M * f.ff].view(M, f.ff)
+        self._lin(d["xb"], Fw.gu, Fw.gu_t, gu)
+        ops.gated_act(gu, h, 1)
+        self._lin(h, Fw.down, Fw.down_t, d["y"])
+
+    @staticmethod
+    def _cols(buf, c0: int, heads: int, width: int):
+        """Columns [c0, c0 + heads * width) of a row-major fp32 buffer as [rows, heads, width] (a view)."""
+        return buf[:, c0:c0 + heads * width].unflatten(1, (heads, width))
+
+    def _scan_out(self, ri: int, Lw_norm, gate, H: int, V: int, M: int, d: dict, q, k, v, decay, beta, groups, q_scale,
+                  o_w, o_t, y) -> None:
+        """Recurrence over every sequence group, per-head output norm times the SiLU gate, output projection."""
+        o = d["o"][:M * H * V].view(M, H, V)
+        for g in groups:
+            ops.matrix_scan(q, k, v, decay, beta, self.state.state[ri], g["qs"], g["ql"], g["ctx"], g["ss"], o, q_scale)
+        ao = d["ao"][:M * H * V].view(M, H * V)
+        ops.gated_head_norm(o, Lw_norm, gate, self.cfg.eps, ao)
+        self._lin(ao, o_w, o_t, y)
+
+    def _delta(self, ri: int, m, Lw, M: int, d: dict, pos, slots, groups: list) -> None:
+        H, G, D, V = m.heads, m.kv_heads, m.dim, m.vdim
+        C = 2 * G * D + H * V
+        big = d["big"][:M * (C + H * V)].view(M, C + H * V)
+        small = d["small"][:M * 2 * H].view(M, 2 * H)
+        cv = d["cv"][:M * C].view(M, C)
+        self._lin(d["xb"], Lw.big, Lw.big_t, big)
+        ops.gemm_rm(d["xb"], Lw.small, small)
+        for g in groups:
+            ops.conv_state(big[:, :C], Lw.conv, None, self.state.tail.get(ri), g["qs"], g["ql"], g["ctx"], g["ss"], cv,
+                           None, None, 1)
+        q, k, v = self._cols(cv, 0, G, D), self._cols(cv, G * D, G, D), self._cols(cv, 2 * G * D, H, V)
+        ops.norm_rope_rows(q, None, pos, None, q, None, 2, UNIT_EPS, D ** -0.5)
+        ops.norm_rope_rows(k, None, pos, None, k, None, 2, UNIT_EPS, 1.0)
+        ops.gate_math(small[:, :H], 0, Lw.a_log, Lw.dt_bias)
+        ops.gate_math(small[:, H:], 1)
+        self._scan_out(ri, Lw.norm, big[:, C:], H, V, M, d, q, k, v, small[:, :H], small[:, H:], groups, 1.0, Lw.o,
+                       Lw.o_t, d["y"])
+
+    def _parallel(self, ri: int, m, Lw, M: int, d: dict, pos, slots, groups: list) -> None:
+        a, r = m.left, m.right
+        H, G, D, V = a.heads, a.kv_heads, a.dim, a.vdim
+        Hr, Dr, Vr = r.heads, r.dim, r.vdim
+        NL, NR = (H + G) * D + G * V, 2 * Hr * (Dr + Vr)
+        rank = Lw.a2.shape[1]
+        big = d["big"][:M * (NL + NR)].view(M, NL + NR)
+        small = d["small"][:M * (H + rank)].view(M, H + rank)
+        self._lin(d["xb"], Lw.big, Lw.big_t, big)
+        ops.gemm_rm(d["xb"], Lw.small, small)
+        # left: softmax attention with a sink over this run's pages
+        rope = self._rope.get(a.rot)
+        qa = d["qa"][:M * H * D].view(M, H, D)
+        ops.norm_rope_rows(self._cols(big, 0, H, D), Lw.q_norm, pos, rope, qa, None, 1, self.cfg.eps, 1.0)
+        ops.norm_rope_rows(self._cols(big, H * D, G, D), Lw.k_norm, pos, rope, self.kv.k[ri], slots, 1, self.cfg.eps, 1.0)
+        ops.norm_rope_rows(self._cols(big, (H + G) * D, G, V), None, pos, None, self.kv.v[ri], slots, 0, 0.0, 1.0)
+        ao = d["ao"][:M * H * V].view(M, H, V)
+        for g in groups:
+            ops.sink_attention(qa, self.kv.k[ri], self.kv.v[ri], g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"], g["wt"],
+                               Lw.sink, small[:, :H], ao, a.window, a.scale, g["qt"])
+        self._lin(ao.view(M, H * V), Lw.lo, Lw.lo_t, d["y"])
+        # right: gated linear attention, decay per key channel from the low-rank projection (fp32 throughout)
+        z = d["z"][:M * Hr * Dr].view(M, Hr * Dr)
+        ops.gemm_rm(small[:, H:], Lw.a2, z, bias=Lw.a2_b)
+        ops.gate_math(z, 2, None, None, r.tau)
+        c0 = NL
+        q, k = self._cols(big, c0, Hr, Dr), self._cols(big, c0 + Hr * Dr, Hr, Dr)
+        v = self._cols(big, c0 + 2 * Hr * Dr, Hr, Vr)
+        gate = big[:, c0 + 2 * Hr * Dr + Hr * Vr:]
+        self._scan_out(ri, Lw.rnorm, gate, Hr, Vr, M, d, q, k, v, z.view(M, Hr, Dr), None, groups, Dr ** -0.5, Lw.ro,
+                       Lw.ro_t, d["y2"])
+        ops.rms_mix(d["y"], Lw.left_out, d["y2"], Lw.right_out, self.cfg.eps, 0.5, d["y"])
+
+    def _retention(self, ri: int, m, Lw, M: int, d: dict, pos, slots, groups: list) -> None:
+        H, D, V = m.heads, m.dim, m.vdim
+        N = 2 * H * (D + V)
+        big = d["big"][:M * N].view(M, N)
+        self._lin(d["xb"], Lw.big, Lw.big_t, big)
+        rope = self._rope.get(m.rot)
+        q, k, v = self._cols(big, 0, H, D), self._cols(big, H * D, H, D), self._cols(big, 2 * H * D, H, V)
+        ops.norm_rope_rows(q, None, pos, rope, q, None, 0, 0.0, 1.0)
+        ops.norm_rope_rows(k, None, pos, rope, k, None, 0, 0.0, D ** -0.5)
+        self._scan_out(ri, None, big[:, 2 * H * D + H * V:], H, V, M, d, q, k, v, Lw.decay, None, groups, 1.0, Lw.o,
+                       Lw.o_t, d["y"])
 
     # ------------------------------------------------------------------ decode
     def _decode_group(self, B: int) -> dict:
@@ -234,11 +425,9 @@ class LayeredRunner(RunnerBase):
         r = slice(0, B)
         ops.decode_prep(self.active[r], self.positions[r], self.block_tables[r], self.slots[r], self.ctx_len[r],
                         self.q_len[r], self.kv.num_blocks)
-        d = {k: (v[:B] if k in ("resid", "xb", "y") else v) for k, v in self._dec.items()}
+        d = {k: (v[:B] if k in ("resid", "xb", "y", "y2") else v) for k, v in self._dec.items()}
         self._layers(B, d, self.ids[r], self.positions[r], self.slots[r], [self._decode_group(B)])
-        xn = self._dec["xb"][:B]
-        ops.scalar_norm(None, self.w.final_norm, d["resid"], xn, self.cfg.eps)
-        self._lin(xn, self.w.head, self.w.head_t, self.logits[r])
+        self._head(d["resid"], self._dec["xb"][:B], self.logits[r])
         self._sample_commit(B)
         ops.ring_advance(self.ring_counter)
 

@@ -258,6 +258,7 @@ class LayeredWeights:
     tp_rank: int = 0
     tp_size: int = 1
     head_t: torch.Tensor = None  # the head in the tiled layout when its shape fits (head then None)
+    step: torch.Tensor = None    # [passes, W] fp32: the vector added before each pass of a looped span (or None)
 
     @property
     def vocab_local(self) -> int:
@@ -269,15 +270,18 @@ class LayeredWeights:
 
     def nbytes(self) -> int:
         seen, n = set(), 0
+
+        def size(obj) -> int:
+            if isinstance(obj, torch.Tensor):
+                return obj.numel() * obj.element_size()
+            if obj is None or id(obj) in seen or not hasattr(obj, "__dataclass_fields__"):
+                return 0
+            seen.add(id(obj))
+            return sum(size(v) for v in vars(obj).values())
+
         for L in self.layers:
-            if id(L) in seen:
-                continue
-            seen.add(id(L))
-            for obj in (L, L.mix, L.mlp):
-                if obj is not None:
-                    n += sum(t.numel() * t.element_size() for t in vars(obj).values() if isinstance(t, torch.Tensor))
-        return n + sum(t.numel() * t.element_size() for t in (self.embed, self.final_norm, self.head, self.head_t)
-                       if t is not None)
+            n += size(L)
+        return n + sum(size(t) for t in (self.embed, self.final_norm, self.head, self.head_t, self.step))
 
 
 TILED_MIN = 1024  # smallest N and K that go to the tiled-layout GEMMs
@@ -361,3 +365,142 @@ def load_layered_dir(cfg, path: str, device="cpu", dtype=torch.bfloat16) -> Laye
     for f in sorted(Path(path).glob("*.safetensors")):
         tensors.update(load_file(str(f)))
     return convert_layered(cfg, tensors, device=device, dtype=dtype)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Pre-norm designs with matrix-state mixers (models/surodra.py): every projection that reads the same input is ONE
+# weight (its outputs are column ranges of one fp32 GEMM output); the few-row projections (gates per head, the decay's
+# inner projection) are grouped into a second, small one so that the large one keeps an aligned row count.  Norm gains,
+# sinks and decay parameters are fp32 in both element types.
+@dataclass
+class TanhNormWeights:
+    alpha: torch.Tensor      # [1] fp32
+    w: torch.Tensor          # [W] fp32
+    b: torch.Tensor          # [W] fp32
+
+
+@dataclass
+class DeltaWeights:
+    big: torch.Tensor        # rows [q (G D) | k (G D) | v (H V) | g (H V)] x W
+    small: torch.Tensor      # rows [a (H) | b (H)] x W
+    conv: torch.Tensor       # [2 G D + H V, taps] fp32: the taps of q | k | v
+    a_log: torch.Tensor      # [H] fp32
+    dt_bias: torch.Tensor    # [H] fp32
+    norm: torch.Tensor       # [V] fp32
+    o: torch.Tensor          # [W, H V]
+    big_t: torch.Tensor = None
+    o_t: torch.Tensor = None
+
+
+@dataclass
+class ParallelWeights:
+    big: torch.Tensor        # rows [left q | left k | left v | right q | right k | right v | right g] x W
+    small: torch.Tensor      # rows [left g (H) | right a1 (rank)] x W
+    q_norm: torch.Tensor     # fp32
+    k_norm: torch.Tensor
+    sink: torch.Tensor       # [H] fp32
+    a2: torch.Tensor         # [Hr Dr, rank] fp32 (its input is the fp32 output of a1)
+    a2_b: torch.Tensor       # [Hr Dr] fp32
+    rnorm: torch.Tensor      # [Vr] fp32
+    lo: torch.Tensor         # [W, H V]
+    ro: torch.Tensor         # [W, Hr Vr]
+    left_out: torch.Tensor   # [W] fp32
+    right_out: torch.Tensor
+    big_t: torch.Tensor = None
+    lo_t: torch.Tensor = None
+    ro_t: torch.Tensor = None
+
+
+@dataclass
+class RetentionWeights:
+    big: torch.Tensor        # rows [q | k | v | g] x W
+    decay: torch.Tensor      # [H] fp32
+    o: torch.Tensor
+    big_t: torch.Tensor = None
+    o_t: torch.Tensor = None
+
+
+@dataclass
+class DenseFfWeights:
+    gu: torch.Tensor         # rows [gate (F) | up (F)] x W
+    down: torch.Tensor       # [W, F]
+    gu_t: torch.Tensor = None
+    down_t: torch.Tensor = None
+
+
+@dataclass
+class PreNormLayer:
+    norm1: TanhNormWeights
+    mix: object
+    norm2: TanhNormWeights = None
+    mlp: DenseFfWeights = None
+
+
+@torch.no_grad()
+def convert_surodra(cfg, tensors: dict, device="cpu", dtype=torch.bfloat16) -> LayeredWeights:
+    """Checkpoint tensors {name: tensor} (models/surodra.py tensor_shapes) -> the engine's grouped layout in `dtype`."""
+    from ..models.surodra import ANY, tensor_shapes
+
+    for name, shape in tensor_shapes(cfg).items():
+        if name not in tensors:
+            raise KeyError(f"checkpoint lacks tensor {name!r}")
+        got = tuple(tensors[name].shape)
+        if len(got) != len(shape) or any(s != ANY and s != g for s, g in zip(shape, got)):
+            raise ValueError(f"tensor {name!r} has shape {got}, the configuration says {shape}")
+
+    def t(name):
+        return tensors[name].to(device=device, dtype=dtype).contiguous()
+
+    def f(name):
+        return tensors[name].to(device=device, dtype=torch.float32).contiguous()
+
+    def cat(*names):
+        return torch.cat([t(n) for n in names], dim=0).contiguous()
+
+    def norm(name):
+        return TanhNormWeights(alpha=f(name + ".alpha").reshape(1), w=f(name), b=f(name + ".b"))
+
+    layers = []
+    for i, L in enumerate(cfg.layers):
+        p = f"l{i}.mix."
+        if L.kind == "delta":
+            mix = DeltaWeights(big=cat(p + "q", p + "k", p + "v", p + "g"), small=cat(p + "a", p + "b"),
+                               conv=torch.cat([f(p + "q.conv"), f(p + "k.conv"), f(p + "v.conv")]).contiguous(),
+                               a_log=f(p + "A_log"), dt_bias=f(p + "dt_bias"), norm=f(p + "norm"), o=t(p + "o"))
+            _tile_fields(mix, ("big", "o"))
+        elif L.kind == "parallel":
+            l, r = p + "left.", p + "right."
+            if tensors[r + "a2"].shape[1] != tensors[r + "a1"].shape[0]:
+                raise ValueError(f"layer {i}: the decay's two projections disagree on their inner width")
+            mix = ParallelWeights(big=cat(l + "q", l + "k", l + "v", r + "q", r + "k", r + "v", r + "g"),
+                                  small=cat(l + "g", r + "a1"), q_norm=f(l + "q.norm"), k_norm=f(l + "k.norm"),
+                                  sink=f(l + "sink"), a2=f(r + "a2"), a2_b=f(r + "a2.b"), rnorm=f(r + "norm"),
+                                  lo=t(l + "o"), ro=t(r + "o"), left_out=f(l + "out"), right_out=f(r + "out"))
+            _tile_fields(mix, ("big", "lo", "ro"))
+        else:
+            mix = RetentionWeights(big=cat(p + "q", p + "k", p + "v", p + "g"),
+                                   decay=torch.tensor(L.mixer.decay, dtype=torch.float32, device=device), o=t(p + "o"))
+            _tile_fields(mix, ("big", "o"))
+        layer = PreNormLayer(norm1=norm(f"l{i}.norm1"), mix=mix)
+        if L.mlp is not None:
+            layer.norm2 = norm(f"l{i}.norm2")
+            layer.mlp = DenseFfWeights(gu=cat(f"l{i}.mlp.gate", f"l{i}.mlp.up"), down=t(f"l{i}.mlp.down"))
+            _tile_fields(layer.mlp, ("gu", "down"))
+        layers.append(layer)
+    out = LayeredWeights(cfg=cfg, embed=t("embed"), layers=layers, final_norm=norm("final.norm"), head=t("head"),
+                         dtype=dtype)
+    out.step = f("loop.step") if cfg.loop_times > 0 else None
+    _tile_fields(out, ("head",))
+    return out
+
+
+def load_surodra_dir(cfg, path: str, device="cpu", dtype=torch.bfloat16) -> LayeredWeights:
+    """``*.safetensors`` of a checkpoint directory -> the engine's layout (the loader executes nothing from the files)."""
+    from pathlib import Path
+
+    from safetensors.torch import load_file
+
+    tensors = {}
+    for f in sorted(Path(path).glob("*.safetensors")):
+        tensors.update(load_file(str(f)))
+    return convert_surodra(cfg, tensors, device=device, dtype=dtype)

@@ -79,13 +79,14 @@ def latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, wor
                               window, scale, qt, vt)
 
 
-def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias=None):
+def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias=None, act: int = 0):
     """Per-channel causal convolution continued from each sequence's slot tail (and the tail's update); in_bias is
-    added to every input (the bias of the projection that made `inp`)."""
+    added to every input (the bias of the projection that made `inp`).  `inp` may be a column slice of a wider fp32
+    buffer; bias and out_b (the output once more in the element type) may be None; act 1 applies SiLU to the output."""
     if _hip(inp):
-        torch.ops.dsse.conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias)
+        torch.ops.dsse.conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias, act)
     else:
-        lref.conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias)
+        lref.conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias, act)
 
 
 def lru_scan(u, gates, y, lam, state, q_start, q_len, ctx_len, state_slot, out, c: float, y_bias=None,
@@ -134,3 +135,89 @@ def moe_grouped(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, sorted_i
                                    num_tiles, h, o)
     else:
         lref.moe_grouped(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, o)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Pre-norm designs with matrix-state mixers.  Small parameter vectors (norm gains, sinks, decay parameters) are fp32
+# in both element types.
+def stream_step(y, mult: float, resid, ids, embed, vec, alpha, w, b, xb):
+    """The residual stream's step between sublayers: resid (fp32) += mult * y (y given) + embed[ids] (embed given) +
+    vec (vec [W] given); then, when a norm follows (w given), xb = tanh(alpha * resid) * w + b in the element type."""
+    if _hip(resid):
+        torch.ops.dsse.stream_step(y, mult, resid, ids, embed, vec, alpha, w, b, xb)
+    else:
+        lref.stream_step(y, mult, resid, ids, embed, vec, alpha, w, b, xb)
+
+
+def gated_act(gu, h, kind: int = 1):
+    """h = act(gu[:, :F]) * gu[:, F:] for the fused gate | up projection's fp32 output; kind 0 SiLU, 1 gelu (tanh)."""
+    if _hip(gu):
+        torch.ops.dsse.gated_act(gu, h, kind)
+    else:
+        lref.gated_act(gu, h, kind)
+
+
+def norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind: int, eps: float, scale: float = 1.0):
+    """Rows x [T, heads, D] (fp32, may be a column slice of a wider buffer) -> out rows out_rows[t] (or t) in out's
+    type: an optional norm (1: RMS over the whole row times norm_w; 2: unit vector per head), the rotate-half rotation
+    of the leading 2 * rope.shape[1] coordinates (rope [positions, dims / 2, 2] or None), times scale.  With out_rows =
+    cache rows this writes keys or values straight into their pages."""
+    if _hip(x):
+        torch.ops.dsse.norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind, eps, scale)
+    else:
+        lref.norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind, eps, scale)
+
+
+def sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile, sink, gate, out,
+                   window: int, scale: float, qt: int):
+    """Causal softmax attention of q [T, H, D] over paged keys [pages, 32, G, D] and values [pages, 32, G, V] (grouped
+    heads), scores and weights in fp32; sink [H] adds exp(sink) to each head's denominator, gate [T, H] multiplies the
+    head's output by its sigmoid.  `qt` query rows per work item (work_seq, work_tile)."""
+    if _hip(q):
+        torch.ops.dsse.sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile,
+                                      sink, gate, out, window, scale, qt)
+    else:
+        lref.sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, sink, gate, out, window, scale)
+
+
+def gate_math(x, kind: int, p1=None, p2=None, c: float = 1.0):
+    """In place on fp32 x [T, N] (a column slice is fine): 0: exp(-exp(p1) * softplus(x + p2)); 1: sigmoid(x);
+    2: sigmoid(x)^(1 / c)."""
+    if _hip(x):
+        torch.ops.dsse.gate_math(x, kind, p1, p2, c)
+    else:
+        lref.gate_math(x, kind, p1, p2, c)
+
+
+def matrix_scan(q, k, v, decay, beta, state, q_start, q_len, ctx_len, state_slot, out, q_scale: float = 1.0):
+    """Matrix-state recurrence per (sequence, head) continued from the slot state [slots, H, D, V] (fp32; zeros at
+    position 0): S = a S; u = beta (v - S^T k) with beta (the delta rule), else u = v; S += k u^T; o = S^T (q_scale q).
+    decay: None, [H], [T, H] or [T, H, D]; q, k [T, G, D], v [T, H, V] are fp32 (column slices are fine)."""
+    if _hip(v):
+        torch.ops.dsse.matrix_scan(q, k, v, decay, beta, state, q_start, q_len, ctx_len, state_slot, out, q_scale)
+    else:
+        lref.matrix_scan(q, k, v, decay, beta, state, q_start, q_len, ctx_len, state_slot, out, q_scale)
+
+
+def gated_head_norm(o, w, gate, eps: float, out):
+    """out [T, H * V] (element type) = o / rms(o) per head * w (or no gain) * silu(gate)."""
+    if _hip(o):
+        torch.ops.dsse.gated_head_norm(o, w, gate, eps, out)
+    else:
+        lref.gated_head_norm(o, w, gate, eps, out)
+
+
+def rms_mix(ya, wa, yb, wb, eps: float, coef: float, out):
+    """out (fp32) = coef * (rms-norm(ya) * wa + rms-norm(yb) * wb)."""
+    if _hip(ya):
+        torch.ops.dsse.rms_mix(ya, wa, yb, wb, eps, coef, out)
+    else:
+        lref.rms_mix(ya, wa, yb, wb, eps, coef, out)
+
+
+def logit_cap(logits, scale: float, cap: float):
+    """In place: logits * scale, then cap * tanh(. / cap) when cap > 0."""
+    if _hip(logits):
+        torch.ops.dsse.logit_cap(logits, scale, cap)
+    else:
+        lref.logit_cap(logits, scale, cap)

@@ -104,7 +104,8 @@ def latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, wor
             out[row] = (p @ val).to(out.dtype)
 
 
-def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias=None):
+def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias=None, act=0):
+    """inp may be a column slice of a wider buffer; act 1: SiLU on the output (the tail keeps raw inputs)."""
     K = taps.shape[1]
     tp = taps.float()
     ib = 0.0 if in_bias is None else in_bias.float()
@@ -115,12 +116,15 @@ def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, 
         r0, slot = int(q_start[s]), int(state_slot[s])
         fresh = int(ctx_len[s]) - ql == 0
         prev = torch.zeros(K - 1, inp.shape[1]) if fresh else tail[slot].clone()
-        seq = torch.cat([prev, inp[r0:r0 + ql] + ib])
+        seq = torch.cat([prev, inp[r0:r0 + ql].float() + ib])
         y = torch.zeros(ql, inp.shape[1]) if bias is None else bias.float().expand(ql, -1).clone()
         for k in range(K):
             y = y + seq[k:k + ql] * tp[:, k]
+        if act == 1:
+            y = torch.nn.functional.silu(y)
         out[r0:r0 + ql] = y
-        out_b[r0:r0 + ql] = y.to(out_b.dtype)
+        if out_b is not None:
+            out_b[r0:r0 + ql] = y.to(out_b.dtype)
         if K > 1:
             tail[slot] = seq[ql:]
 
@@ -200,3 +204,159 @@ def moe_grouped(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, o):
             ov[rows, ks] = ffn(xf[rows], gate[e], up[e], down[e]) * topk_w[rows, ks].unsqueeze(-1)
     if sgate is not None:
         ov[:, top] = ffn(xf, sgate, sup, sdown)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Pre-norm designs with matrix-state mixers (models/surodra.py)
+def stream_step(y, mult, resid, ids, embed, vec, alpha, w, b, xb):
+    """resid += mult * y (y given) + embed[ids] (embed given) + vec (vec given); then, with a norm (w given),
+    xb = tanh(alpha * resid) * w + b."""
+    M = resid.shape[0]
+    if y is not None:
+        resid.add_(y.float() * mult)
+    if embed is not None:
+        idx = ids[:M].long()
+        idx = torch.where((idx >= 0) & (idx < embed.shape[0]), idx, torch.zeros_like(idx))
+        resid.add_(embed[idx].float())
+    if vec is not None:
+        resid.add_(vec.float())
+    if w is not None:
+        xb.copy_((torch.tanh(alpha.float().reshape(()) * resid) * w.float() + b.float()).to(xb.dtype))
+
+
+def gated_act(gu, h, kind):
+    """h = act(gu[:, :F]) * gu[:, F:]; kind 0 SiLU, 1 gelu (tanh form)."""
+    F = h.shape[1]
+    g, u = gu[:, :F].float(), gu[:, F:].float()
+    h.copy_(((torch.nn.functional.silu(g) if kind == 0 else gelu_tanh(g)) * u).to(h.dtype))
+
+
+def rotate_half_rows(v, cs, dims):
+    """v [T, heads, D], cs [T, dims / 2, 2]: coordinate i < dims / 2 pairs with i + dims / 2."""
+    half = dims // 2
+    a, b = v[..., :half], v[..., half:dims]
+    c, s = cs[:, None, :, 0], cs[:, None, :, 1]
+    out = v.clone()
+    out[..., :half] = a * c - b * s
+    out[..., half:dims] = b * c + a * s
+    return out
+
+
+def norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind, eps, scale):
+    """x [T, heads, D] fp32 -> out rows (out_rows[t], or t) as [heads, D] in out's type.  norm_kind 1: RMS norm over
+    the whole row (all heads at once) times norm_w [heads * D]; 2: every head divided by sqrt(sum of squares + eps);
+    then the rotate-half rotation of the leading 2 * rope.shape[1] coordinates at positions[t]; then times scale.
+    Rows whose out_rows entry is negative are skipped."""
+    T, nh, D = x.shape
+    v = x.float()
+    if norm_kind == 1:
+        flat = v.reshape(T, nh * D)
+        v = (flat / torch.sqrt(flat.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()).view(T, nh, D)
+    elif norm_kind == 2:
+        v = v / torch.sqrt(v.pow(2).sum(-1, keepdim=True) + eps)
+    if rope is not None and rope.shape[1] > 0:
+        pos = positions[:T].long().clamp(0, rope.shape[0] - 1)
+        v = rotate_half_rows(v, rope[pos], 2 * rope.shape[1])
+    v = (v * scale).to(out.dtype)
+    if out_rows is None:
+        out.copy_(v)
+    else:
+        flat_out = out.view(-1, nh, D)
+        r = out_rows[:T].long()
+        ok = (r >= 0) & (r < flat_out.shape[0])
+        flat_out[r[ok]] = v[ok]
+
+
+def sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, sink, gate, out, window, scale):
+    """Softmax attention over paged keys [pages, PAGE, G, D] and values [pages, PAGE, G, V] with grouped heads; the
+    denominator also holds exp(sink[h]) when sink is given; the head's output is multiplied by sigmoid(gate[row, h])
+    when gate is given."""
+    H = q.shape[1]
+    G = kcache.shape[2]
+    kf = kcache.view(-1, G, kcache.shape[3]).float()
+    vf = vcache.view(-1, G, vcache.shape[3]).float()
+    grp = torch.arange(H) // (H // G)
+    for s in range(q_len.numel()):
+        ql = int(q_len[s])
+        if ql <= 0:
+            continue
+        r0, p0 = int(q_start[s]), int(ctx_len[s]) - ql
+        bt = block_tables[s].long()
+        for i in range(ql):
+            pos = p0 + i
+            j = torch.arange(max(0, pos - window + 1), pos + 1)
+            rows = bt[j // PAGE] * PAGE + j % PAGE
+            k, v = kf[rows][:, grp], vf[rows][:, grp]                       # [keys, H, D], [keys, H, V]
+            sc = torch.einsum("hd,jhd->hj", q[r0 + i].float(), k) * scale
+            mx = sc.max(-1, keepdim=True).values
+            if sink is not None:
+                mx = torch.maximum(mx, sink.float()[:, None])
+            e = torch.exp(sc - mx)
+            den = e.sum(-1, keepdim=True)
+            if sink is not None:
+                den = den + torch.exp(sink.float()[:, None] - mx)
+            o = torch.einsum("hj,jhv->hv", e / den, v)
+            if gate is not None:
+                o = o * torch.sigmoid(gate[r0 + i].float())[:, None]
+            out[r0 + i] = o.to(out.dtype)
+
+
+def gate_math(x, kind, p1, p2, c):
+    """In place on fp32 x [T, N]: kind 0: exp(-exp(p1) * softplus(x + p2)) (p1, p2 [N]); 1: sigmoid(x);
+    2: sigmoid(x)^(1 / c) as exp(logsigmoid(x) / c)."""
+    if kind == 0:
+        x.copy_(torch.exp(-torch.exp(p1.float()) * torch.nn.functional.softplus(x + p2.float())))
+    elif kind == 1:
+        x.copy_(torch.sigmoid(x))
+    else:
+        x.copy_(torch.exp(torch.nn.functional.logsigmoid(x) / c))
+
+
+def matrix_scan(q, k, v, decay, beta, state, q_start, q_len, ctx_len, state_slot, out, q_scale=1.0):
+    """Matrix-state recurrence per (sequence, head), continued from the sequence's slot (zeros at position 0):
+    S = a S; with beta (delta rule) u = beta (v - S^T k) else u = v; S += k u^T; o = S^T q.  q, k [T, G, D] (head h
+    reads group h / (H / G)), v [T, H, V], state [slots, H, D, V] fp32, out [T, H, V] fp32.  decay: None, [H] (fixed
+    per head), [T, H] (per row and head) or [T, H, D] (per row, head and key channel).  q is multiplied by q_scale."""
+    T, H, V = v.shape
+    G, D = k.shape[1], k.shape[2]
+    grp = torch.arange(H) // (H // G)
+    for s in range(q_len.numel()):
+        ql = int(q_len[s])
+        if ql <= 0:
+            continue
+        r0, slot = int(q_start[s]), int(state_slot[s])
+        S = torch.zeros(H, D, V) if int(ctx_len[s]) - ql == 0 else state[slot].clone()
+        for t in range(r0, r0 + ql):
+            kt, qt, vt = k[t].float()[grp], q[t].float()[grp] * q_scale, v[t].float()
+            if decay is not None:
+                a = decay.float() if decay.dim() == 1 else decay[t].float()
+                S = S * (a[:, None, None] if a.dim() == 1 else a[:, :, None])
+            if beta is not None:
+                vt = beta[t].float()[:, None] * (vt - torch.einsum("hdv,hd->hv", S, kt))
+            S = S + kt[:, :, None] * vt[:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", S, qt)
+        state[slot] = S
+
+
+def gated_head_norm(o, w, gate, eps, out):
+    """out [T, H * V] = o / rms(o over V) * w (w [V] or None) * silu(gate [T, H * V])."""
+    T, H, V = o.shape
+    n = o.float() / torch.sqrt(o.float().pow(2).mean(-1, keepdim=True) + eps)
+    if w is not None:
+        n = n * w.float()
+    out.copy_((n.reshape(T, H * V) * torch.nn.functional.silu(gate.float())).to(out.dtype))
+
+
+def rms_mix(ya, wa, yb, wb, eps, coef, out):
+    """out (fp32) = coef * (ya / rms(ya) * wa + yb / rms(yb) * wb), rows of the model width."""
+    def n(y, w):
+        return y.float() / torch.sqrt(y.float().pow(2).mean(-1, keepdim=True) + eps) * w.float()
+
+    out.copy_(coef * (n(ya, wa) + n(yb, wb)))
+
+
+def logit_cap(logits, scale, cap):
+    """In place: logits *= scale; with cap > 0 then cap * tanh(logits / cap)."""
+    logits.mul_(scale)
+    if cap > 0:
+        logits.copy_(cap * torch.tanh(logits / cap))
