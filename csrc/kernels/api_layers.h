@@ -73,7 +73,7 @@ struct LatentAttnParams {
 };
 
 struct ConvStateParams {
-  const float* in;       // [T, C] fp32
+  const float* in;       // [T, C] fp32, rows ld_in apart
   const void* taps;      // [C, K]; taps[c][K - 1] weighs the newest input
   const void* bias;      // [C]
   const void* in_bias;   // [C] or null: added to every input (the input projection's bias; tails hold biased inputs)
@@ -83,9 +83,11 @@ struct ConvStateParams {
   const int* ctx_len;
   const int* state_slot;
   float* out;            // [T, C] fp32
-  void* out_b;           // [T, C] element type (the gates' GEMM input)
+  void* out_b;           // [T, C] element type (the gates' GEMM input) or null
   int nseq, C, K, rows;  // rows = T
   int f32;
+  int ld_in;             // row stride of `in` (a column slice of a wider buffer), C when contiguous
+  int act;               // 0 none, 1 SiLU on the output (the tail keeps the raw inputs)
 };
 
 struct LruScanParams {

@@ -1,0 +1,95 @@
+// Host-visible API of the kernels that serve pre-norm designs with matrix-state mixers: the residual stream's step with
+// the element-wise tanh norm, the gated activation of a fused gate | up projection, per-row norms with the rotate-half
+// rotation (also the write of keys and values into their pages), softmax attention with a sink over paged keys and
+// values of any head width, the gate math of decays, the matrix-state recurrence (plain, decayed, delta rule), the
+// per-head output norm with its SiLU gate, the normed mix of two mixers, and the logit scale and cap.
+//
+// Activations between these kernels are fp32; `T` is the engine's element type (bf16 for serving, fp32 for the exact
+// mode) and appears only where a projection reads or a page stores.  Small parameter vectors are fp32 in both modes.
+// Sequence metadata as in api_layers.h: per sequence q_start, q_len (0 = inactive), ctx_len (tokens after this step).
+#pragma once
+#include "api.h"
+
+namespace dsse {
+
+struct StreamStepParams {
+  const float* y;        // [M, W] sublayer output or null
+  float mult;            // resid += mult * y
+  float* resid;          // [M, W] fp32 stream
+  const int* ids;        // [M] token ids (with embed)
+  const void* embed;     // [vocab, W] element type or null: resid += embed[ids]
+  int vocab;
+  const float* vec;      // [W] or null: resid += vec
+  const float* alpha;    // one number
+  const float* w;        // [W] or null: no norm, xb untouched
+  const float* b;        // [W]
+  void* xb;              // [M, W] element type: tanh(alpha * resid) * w + b
+  int M, W;
+  int f32;
+};
+
+struct NormRopeParams {
+  const float* x;        // [T, nh, D], rows ldx apart
+  const float* norm_w;   // [nh * D] (kind 1) or null
+  const int* positions;  // [T]
+  const float2* rope;    // [rope_len, half] (cos, sin) or null
+  void* out;             // rows ldo apart, [nh, D] each; fp32 when out_f32 else bf16
+  const int* out_rows;   // [T] or null (row t); negative = skip
+  int T, nh, D, ldx, ldo, half, rope_len, num_out_rows;
+  int kind;              // 0 none, 1 RMS over the whole row times norm_w, 2 unit vector per head
+  float eps, scale;
+  int out_f32;
+};
+
+struct SinkAttnParams {
+  const float* q;        // [T, H, D] fp32 (normed, rotated)
+  const void* k;         // [pages * kBS, G, D] element type
+  const void* v;         // [pages * kBS, G, V]
+  const int* block_tables;
+  int max_blocks, num_blocks;
+  const int* q_start;
+  const int* q_len;
+  const int* ctx_len;
+  const int* work_seq;
+  const int* work_tile;
+  const float* sink;     // [H] or null
+  const float* gate;     // [T, ..] rows ldg apart, column h: output times sigmoid, or null
+  void* out;             // [T, H, V] element type
+  int H, G, D, V, window, qt, ldg;
+  float scale;
+  int f32;
+};
+
+struct MatrixScanParams {
+  const float* q;        // [T, G, D] rows ldq apart
+  const float* k;        // rows ldk apart
+  const float* v;        // [T, H, V] rows ldv apart
+  const float* decay;    // kind 1: [H]; 2: [T, H] rows ldd apart; 3: [T, H, D] rows ldd apart
+  const float* beta;     // [T, H] rows ldb apart, or null (no delta rule)
+  float* state;          // [slots, H, D, V]
+  const int* q_start;
+  const int* q_len;
+  const int* ctx_len;
+  const int* state_slot;
+  float* out;            // [T, H, V]
+  int nseq, H, G, D, V, ldq, ldk, ldv, ldd, ldb;
+  int decay_kind;        // 0 none
+  float q_scale;
+};
+
+}  // namespace dsse
+
+extern "C" {
+hipError_t dsse_stream_step(const dsse::StreamStepParams* p, hipStream_t st);
+hipError_t dsse_gated_act(const float* gu, int ldg, void* h, int M, int F, int kind, int f32, hipStream_t st);
+hipError_t dsse_norm_rope_rows(const dsse::NormRopeParams* p, hipStream_t st);
+hipError_t dsse_sink_attention(int num_work, const dsse::SinkAttnParams* p, hipStream_t st);
+hipError_t dsse_gate_math(float* x, int ld, int M, int N, int kind, const float* p1, const float* p2, float c,
+                          hipStream_t st);
+hipError_t dsse_matrix_scan(const dsse::MatrixScanParams* p, hipStream_t st);
+hipError_t dsse_gated_head_norm(const float* o, const float* w, const float* gate, int ldg, void* out, int M, int H,
+                                int V, float eps, int f32, hipStream_t st);
+hipError_t dsse_rms_mix(const float* ya, const float* wa, const float* yb, const float* wb, float* out, int M, int W,
+                        float eps, float coef, hipStream_t st);
+hipError_t dsse_logit_cap(float* logits, long long n, float scale, float cap, hipStream_t st);
+}

@@ -244,21 +244,32 @@ void seq_meta(const Tensor& q_start, const Tensor& q_len, const Tensor& ctx_len,
               "sequence metadata too short");
 }
 
-void conv_state(const Tensor& in, const Tensor& taps, const OptTensor& bias, Tensor& tail, const Tensor& q_start,
-                const Tensor& q_len, const Tensor& ctx_len, const Tensor& state_slot, Tensor& out, Tensor& out_b,
-                const OptTensor& in_bias) {
-  f32t(in, "in");
+void conv_state(const Tensor& in, const Tensor& taps, const OptTensor& bias, const OptTensor& tail, const Tensor& q_start,
+                const Tensor& q_len, const Tensor& ctx_len, const Tensor& state_slot, Tensor& out, const OptTensor& out_b,
+                const OptTensor& in_bias, int64_t act) {
+  gpu(in, "in", false);
+  TORCH_CHECK(in.scalar_type() == at::kFloat, "in must be fp32");
   gpu(taps, "taps");
-  f32t(tail, "tail");
   f32t(out, "out");
-  gpu(out_b, "out_b");
-  same(taps, out_b, "out_b");
   dsse::ConvStateParams p{};
   seq_meta(q_start, q_len, ctx_len, state_slot, p.nseq);
+  TORCH_CHECK(in.dim() == 2 && taps.dim() == 2, "in must be [T, C], taps [C, K]");
   const int C = (int)in.size(1), K = (int)taps.size(1);
-  TORCH_CHECK(in.dim() == 2 && taps.dim() == 2 && taps.size(0) == C && K >= 1, "taps must be [C, K]");
-  TORCH_CHECK(out.sizes() == in.sizes() && out_b.sizes() == in.sizes(), "out / out_b must match in");
-  TORCH_CHECK(tail.dim() == 3 && tail.size(1) == K - 1 && tail.size(2) == C, "tail must be [slots, K - 1, C]");
+  TORCH_CHECK(taps.size(0) == C && K >= 1, "taps must be [C, K]");
+  TORCH_CHECK(C == 1 || in.stride(1) == 1, "in needs a unit innermost stride");
+  TORCH_CHECK(out.sizes() == in.sizes(), "out must match in");
+  if (out_b.has_value()) {
+    gpu(*out_b, "out_b");
+    same(taps, *out_b, "out_b");
+    TORCH_CHECK(out_b->sizes() == in.sizes(), "out_b must match in");
+    p.out_b = out_b->data_ptr();
+  }
+  if (K > 1) {
+    TORCH_CHECK(tail.has_value(), "a convolution with more than one tap needs its tail");
+    f32t(*tail, "tail");
+    TORCH_CHECK(tail->dim() == 3 && tail->size(1) == K - 1 && tail->size(2) == C, "tail must be [slots, K - 1, C]");
+    p.tail = tail->data_ptr<float>();
+  }
   if (bias.has_value()) {
     gpu(*bias, "bias");
     same(taps, *bias, "bias");
@@ -267,13 +278,11 @@ void conv_state(const Tensor& in, const Tensor& taps, const OptTensor& bias, Ten
   }
   p.in = in.data_ptr<float>();
   p.taps = taps.data_ptr();
-  p.tail = tail.data_ptr<float>();
   p.q_start = q_start.data_ptr<int>();
   p.q_len = q_len.data_ptr<int>();
   p.ctx_len = ctx_len.data_ptr<int>();
   p.state_slot = state_slot.data_ptr<int>();
   p.out = out.data_ptr<float>();
-  p.out_b = out_b.data_ptr();
   if (in_bias.has_value()) {
     gpu(*in_bias, "in_bias");
     same(taps, *in_bias, "in_bias");
@@ -281,6 +290,9 @@ void conv_state(const Tensor& in, const Tensor& taps, const OptTensor& bias, Ten
     p.in_bias = in_bias->data_ptr();
   }
   p.C = C, p.K = K, p.rows = (int)in.size(0);
+  p.ld_in = (int)in.stride(0);
+  TORCH_CHECK(act == 0 || act == 1, "act: 0 none, 1 SiLU");
+  p.act = (int)act;
   TORCH_CHECK(p.nseq <= 65535 && (p.rows + 31) / 32 <= 65535, "conv_state: grid too large");
   p.f32 = elem(taps, "taps");
   DSSE_CHECK_HIP(dsse_conv_state(&p, cur_stream()));
@@ -505,8 +517,8 @@ TORCH_LIBRARY_FRAGMENT(dsse, m) {
   m.def("latent_attention(Tensor q, Tensor q_abs, Tensor cache, Tensor block_tables, Tensor q_start, Tensor q_len, "
         "Tensor ctx_len, Tensor work_seq, Tensor work_tile, Tensor rope, Tensor(a!) out, int window, float scale, "
         "int qt, Tensor? vt=None, int hp=1, Tensor(b!)? part=None, int nparts=1) -> ()");
-  m.def("conv_state(Tensor inp, Tensor taps, Tensor? bias, Tensor(a!) tail, Tensor q_start, Tensor q_len, "
-        "Tensor ctx_len, Tensor state_slot, Tensor(b!) out, Tensor(c!) out_b, Tensor? in_bias=None) -> ()");
+  m.def("conv_state(Tensor inp, Tensor taps, Tensor? bias, Tensor(a!)? tail, Tensor q_start, Tensor q_len, "
+        "Tensor ctx_len, Tensor state_slot, Tensor(b!) out, Tensor(c!)? out_b, Tensor? in_bias=None, int act=0) -> ()");
   m.def("lru_scan(Tensor u, Tensor(c!) gates, Tensor y, Tensor lam, Tensor(a!) state, Tensor q_start, Tensor q_len, "
         "Tensor ctx_len, Tensor state_slot, Tensor(b!) out, float c, Tensor? y_bias=None, bool coeff=True, "
         "Tensor(d!)? scratch=None) -> ()");

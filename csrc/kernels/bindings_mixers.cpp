@@ -1,0 +1,348 @@
+// torch operator registrations (namespace torch.ops.dsse) of the kernels in api_mixers.h: the residual stream's step
+// with the element-wise tanh norm, the gated activation, per-row norms with rotation, softmax attention with a sink
+// over paged keys and values, gate math, the matrix-state recurrence, the gated per-head output norm, the normed mix
+// of two mixers and the logit cap.
+//
+// As in the other binding files, every op validates device, dtype and the shapes and strides its kernel's indexing
+// assumes before launching, and launches on torch's current HIP stream (graph-capturable).  Column slices of wider
+// fp32 buffers are passed as views (unit innermost stride); nothing is copied here.
+#include <ATen/ATen.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/library.h>
+
+#include <algorithm>
+#include <climits>
+#include <cstdint>
+
+#include "api_mixers.h"
+
+namespace {
+
+using at::Tensor;
+using OptTensor = c10::optional<Tensor>;
+
+hipStream_t cur_stream() { return c10::hip::getCurrentHIPStream().stream(); }
+
+#define DSSE_CHECK_HIP(expr)                                                             \
+  do {                                                                                   \
+    hipError_t _e = (expr);                                                              \
+    TORCH_CHECK(_e == hipSuccess, "dsse kernel launch failed: ", hipGetErrorString(_e)); \
+  } while (0)
+
+void gpu(const Tensor& t, const char* name, bool contiguous = true) {
+  TORCH_CHECK(t.is_cuda(), name, " must be a GPU tensor");
+  if (contiguous) TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
+}
+void i32(const Tensor& t, const char* name) {
+  gpu(t, name);
+  TORCH_CHECK(t.scalar_type() == at::kInt, name, " must be int32");
+}
+void f32t(const Tensor& t, const char* name, bool contiguous = true) {
+  gpu(t, name, contiguous);
+  TORCH_CHECK(t.scalar_type() == at::kFloat, name, " must be fp32");
+}
+int elem(const Tensor& a, const char* name) {
+  TORCH_CHECK(a.scalar_type() == at::kFloat || a.scalar_type() == at::kBFloat16, name, " must be bf16 or fp32");
+  return a.scalar_type() == at::kFloat ? 1 : 0;
+}
+const float* opt_f32(const OptTensor& t, const char* name, int64_t numel) {
+  if (!t.has_value()) return nullptr;
+  f32t(*t, name);
+  TORCH_CHECK(t->numel() == numel, name, " must hold ", numel, " numbers");
+  return t->data_ptr<float>();
+}
+// a [rows, heads, width] fp32 view whose heads are adjacent columns of a row-major buffer
+void head_view(const Tensor& t, const char* name) {
+  f32t(t, name, false);
+  TORCH_CHECK(t.dim() == 3 && (t.size(2) == 1 || t.stride(2) == 1) && (t.size(1) == 1 || t.stride(1) == t.size(2)),
+              name, " must be [rows, heads, width] with adjacent heads");
+  TORCH_CHECK(t.stride(0) >= t.size(1) * t.size(2), name, ": rows overlap");
+}
+// a [rows, cols] fp32 view with a unit innermost stride
+void col_view(const Tensor& t, const char* name) {
+  f32t(t, name, false);
+  TORCH_CHECK(t.dim() == 2 && (t.size(1) == 1 || t.stride(1) == 1) && t.stride(0) >= t.size(1), name,
+              " must be [rows, cols] with a unit innermost stride");
+}
+void seq_meta(const Tensor& q_start, const Tensor& q_len, const Tensor& ctx_len, int ns) {
+  i32(q_start, "q_start");
+  i32(q_len, "q_len");
+  i32(ctx_len, "ctx_len");
+  TORCH_CHECK(q_start.numel() >= ns && q_len.numel() >= ns && ctx_len.numel() >= ns, "sequence metadata too short");
+}
+
+void stream_step(const OptTensor& y, double mult, Tensor& resid, const OptTensor& ids, const OptTensor& embed,
+                 const OptTensor& vec, const OptTensor& alpha, const OptTensor& w, const OptTensor& b,
+                 const OptTensor& xb) {
+  f32t(resid, "resid");
+  TORCH_CHECK(resid.dim() == 2, "resid must be [M, W]");
+  dsse::StreamStepParams p{};
+  p.M = (int)resid.size(0), p.W = (int)resid.size(1);
+  p.resid = resid.data_ptr<float>();
+  p.mult = (float)mult;
+  p.f32 = 1;
+  if (y.has_value()) {
+    f32t(*y, "y");
+    TORCH_CHECK(y->sizes() == resid.sizes(), "y must match resid");
+    p.y = y->data_ptr<float>();
+  }
+  if (embed.has_value()) {
+    TORCH_CHECK(ids.has_value(), "embed needs ids");
+    i32(*ids, "ids");
+    gpu(*embed, "embed");
+    TORCH_CHECK(embed->dim() == 2 && embed->size(1) == p.W && ids->numel() >= p.M, "embed must be [vocab, W]");
+    p.ids = ids->data_ptr<int>();
+    p.embed = embed->data_ptr();
+    p.vocab = (int)embed->size(0);
+    p.f32 = elem(*embed, "embed");
+  }
+  p.vec = opt_f32(vec, "vec", p.W);
+  if (w.has_value()) {
+    TORCH_CHECK(alpha.has_value() && b.has_value() && xb.has_value(), "a norm needs alpha, w, b and xb");
+    p.alpha = opt_f32(alpha, "alpha", 1);
+    p.w = opt_f32(w, "w", p.W);
+    p.b = opt_f32(b, "b", p.W);
+    gpu(*xb, "xb");
+    TORCH_CHECK(xb->sizes() == resid.sizes(), "xb must match resid");
+    const int f = elem(*xb, "xb");
+    TORCH_CHECK(!embed.has_value() || f == p.f32, "embed and xb differ in type");
+    p.f32 = f;
+    p.xb = xb->data_ptr();
+  }
+  DSSE_CHECK_HIP(dsse_stream_step(&p, cur_stream()));
+}
+
+void gated_act(const Tensor& gu, Tensor& h, int64_t kind) {
+  col_view(gu, "gu");
+  gpu(h, "h");
+  TORCH_CHECK(h.dim() == 2 && gu.size(0) == h.size(0) && gu.size(1) == 2 * h.size(1), "gu must be [M, 2 F], h [M, F]");
+  TORCH_CHECK(kind == 0 || kind == 1, "kind: 0 SiLU, 1 gelu");
+  DSSE_CHECK_HIP(dsse_gated_act(gu.data_ptr<float>(), (int)gu.stride(0), h.data_ptr(), (int)h.size(0), (int)h.size(1),
+                                (int)kind, elem(h, "h"), cur_stream()));
+}
+
+void norm_rope_rows(const Tensor& x, const OptTensor& norm_w, const Tensor& positions, const OptTensor& rope, Tensor& out,
+                    const OptTensor& out_rows, int64_t kind, double eps, double scale) {
+  head_view(x, "x");
+  dsse::NormRopeParams p{};
+  p.T = (int)x.size(0), p.nh = (int)x.size(1), p.D = (int)x.size(2);
+  p.ldx = (int)x.stride(0);
+  p.x = x.data_ptr<float>();
+  TORCH_CHECK(kind >= 0 && kind <= 2 && p.D <= 512, "kind 0..2, head width <= 512");
+  p.kind = (int)kind;
+  p.norm_w = opt_f32(norm_w, "norm_w", (int64_t)p.nh * p.D);
+  TORCH_CHECK(kind != 1 || p.norm_w, "kind 1 needs norm_w");
+  if (rope.has_value() && rope->numel() > 0) {
+    f32t(*rope, "rope");
+    i32(positions, "positions");
+    TORCH_CHECK(rope->dim() == 3 && rope->size(2) == 2 && 2 * rope->size(1) <= p.D, "rope must be [P, dims / 2, 2]");
+    TORCH_CHECK(positions.numel() >= p.T, "positions too short");
+    p.rope = reinterpret_cast<const float2*>(rope->data_ptr<float>());
+    p.positions = positions.data_ptr<int>();
+    p.half = (int)rope->size(1), p.rope_len = (int)rope->size(0);
+  }
+  gpu(out, "out", false);
+  TORCH_CHECK(out.scalar_type() == at::kFloat || out.scalar_type() == at::kBFloat16, "out must be fp32 or bf16");
+  p.out_f32 = out.scalar_type() == at::kFloat;
+  p.out = out.data_ptr();
+  if (out_rows.has_value()) {  // out: contiguous rows of [nh, D] (a cache: [pages, page, nh, D])
+    i32(*out_rows, "out_rows");
+    TORCH_CHECK(out.is_contiguous() && out.dim() >= 3 && out.size(-1) == p.D && out.size(-2) == p.nh,
+                "out must be contiguous [..., heads, width]");
+    TORCH_CHECK(out_rows->numel() >= p.T, "out_rows too short");
+    p.out_rows = out_rows->data_ptr<int>();
+    p.ldo = p.nh * p.D;
+    p.num_out_rows = (int)(out.numel() / p.ldo);
+  } else {
+    TORCH_CHECK(out.dim() == 3 && out.sizes() == x.sizes() && (p.D == 1 || out.stride(2) == 1) &&
+                    (p.nh == 1 || out.stride(1) == p.D) && out.stride(0) >= (int64_t)p.nh * p.D,
+                "out must be [rows, heads, width] with adjacent heads");
+    p.ldo = (int)out.stride(0);
+    p.num_out_rows = p.T;
+  }
+  p.eps = (float)eps, p.scale = (float)scale;
+  DSSE_CHECK_HIP(dsse_norm_rope_rows(&p, cur_stream()));
+}
+
+void sink_attention(const Tensor& q, const Tensor& kcache, const Tensor& vcache, const Tensor& block_tables,
+                    const Tensor& q_start, const Tensor& q_len, const Tensor& ctx_len, const Tensor& work_seq,
+                    const Tensor& work_tile, const OptTensor& sink, const OptTensor& gate, Tensor& out, int64_t window,
+                    double scale, int64_t qt) {
+  f32t(q, "q");
+  gpu(kcache, "kcache");
+  gpu(vcache, "vcache");
+  gpu(out, "out");
+  TORCH_CHECK(kcache.scalar_type() == vcache.scalar_type() && out.scalar_type() == kcache.scalar_type(),
+              "kcache, vcache and out share the element type");
+  i32(block_tables, "block_tables");
+  i32(work_seq, "work_seq");
+  i32(work_tile, "work_tile");
+  TORCH_CHECK(q.dim() == 3 && kcache.dim() == 4 && vcache.dim() == 4 && out.dim() == 3, "q [T, H, D], caches 4-D");
+  dsse::SinkAttnParams p{};
+  const int T = (int)q.size(0);
+  p.H = (int)q.size(1), p.D = (int)q.size(2), p.G = (int)kcache.size(2), p.V = (int)vcache.size(3);
+  TORCH_CHECK(kcache.size(1) == dsse::kBS && vcache.size(1) == dsse::kBS && kcache.size(3) == p.D &&
+                  vcache.size(2) == p.G && vcache.size(0) == kcache.size(0),
+              "caches must be [pages, 32, G, D] and [pages, 32, G, V]");
+  TORCH_CHECK(p.G >= 1 && p.H % p.G == 0 && p.D <= 512 && p.V <= 512, "heads must be a multiple of kv heads, widths <= 512");
+  TORCH_CHECK(out.size(0) == T && out.size(1) == p.H && out.size(2) == p.V, "out must be [T, H, V]");
+  TORCH_CHECK(block_tables.dim() == 2, "block_tables must be [seqs, max_blocks]");
+  const int ns = (int)block_tables.size(0);
+  seq_meta(q_start, q_len, ctx_len, ns);
+  TORCH_CHECK(work_tile.numel() == work_seq.numel() && window >= 1 && qt >= 1, "work lists, window >= 1, qt >= 1");
+  TORCH_CHECK(kcache.size(0) * dsse::kBS * p.G < INT_MAX, "cache rows out of range");
+  p.q = q.data_ptr<float>();
+  p.k = kcache.data_ptr();
+  p.v = vcache.data_ptr();
+  p.block_tables = block_tables.data_ptr<int>();
+  p.max_blocks = (int)block_tables.size(1);
+  p.num_blocks = (int)kcache.size(0);
+  p.q_start = q_start.data_ptr<int>();
+  p.q_len = q_len.data_ptr<int>();
+  p.ctx_len = ctx_len.data_ptr<int>();
+  p.work_seq = work_seq.data_ptr<int>();
+  p.work_tile = work_tile.data_ptr<int>();
+  p.sink = opt_f32(sink, "sink", p.H);
+  if (gate.has_value()) {
+    col_view(*gate, "gate");
+    TORCH_CHECK(gate->size(0) == T && gate->size(1) == p.H, "gate must be [T, H]");
+    p.gate = gate->data_ptr<float>();
+    p.ldg = (int)gate->stride(0);
+  }
+  p.out = out.data_ptr();
+  p.window = (int)std::min<int64_t>(window, INT_MAX), p.qt = (int)qt;
+  p.scale = (float)scale;
+  p.f32 = elem(kcache, "kcache");
+  DSSE_CHECK_HIP(dsse_sink_attention((int)work_seq.numel(), &p, cur_stream()));
+}
+
+void gate_math(Tensor& x, int64_t kind, const OptTensor& p1, const OptTensor& p2, double c) {
+  col_view(x, "x");
+  const int M = (int)x.size(0), N = (int)x.size(1);
+  TORCH_CHECK(kind >= 0 && kind <= 2, "kind 0..2");
+  const float* a = opt_f32(p1, "p1", N);
+  const float* b = opt_f32(p2, "p2", N);
+  TORCH_CHECK(kind != 0 || (a && b), "kind 0 needs p1 and p2");
+  TORCH_CHECK(kind != 2 || c > 0, "kind 2 needs c > 0");
+  DSSE_CHECK_HIP(dsse_gate_math(x.data_ptr<float>(), (int)x.stride(0), M, N, (int)kind, a, b, (float)c, cur_stream()));
+}
+
+void matrix_scan(const Tensor& q, const Tensor& k, const Tensor& v, const OptTensor& decay, const OptTensor& beta,
+                 Tensor& state, const Tensor& q_start, const Tensor& q_len, const Tensor& ctx_len,
+                 const Tensor& state_slot, Tensor& out, double q_scale) {
+  head_view(q, "q");
+  head_view(k, "k");
+  head_view(v, "v");
+  f32t(state, "state");
+  f32t(out, "out");
+  dsse::MatrixScanParams p{};
+  const int T = (int)v.size(0);
+  p.H = (int)v.size(1), p.V = (int)v.size(2), p.G = (int)k.size(1), p.D = (int)k.size(2);
+  TORCH_CHECK(q.sizes() == k.sizes() && q.size(0) == T && p.G >= 1 && p.H % p.G == 0, "q, k [T, G, D], v [T, H, V]");
+  TORCH_CHECK(p.D <= 512, "key width <= 512");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == p.H && state.size(2) == p.D && state.size(3) == p.V,
+              "state must be [slots, H, D, V]");
+  TORCH_CHECK(out.dim() == 3 && out.sizes() == v.sizes(), "out must be [T, H, V]");
+  p.nseq = (int)q_len.numel();
+  seq_meta(q_start, q_len, ctx_len, p.nseq);
+  i32(state_slot, "state_slot");
+  TORCH_CHECK(state_slot.numel() >= p.nseq && p.nseq <= 65535 && p.H <= 65535, "state_slot too short / grid too large");
+  p.q = q.data_ptr<float>(), p.k = k.data_ptr<float>(), p.v = v.data_ptr<float>();
+  p.ldq = (int)q.stride(0), p.ldk = (int)k.stride(0), p.ldv = (int)v.stride(0);
+  if (decay.has_value()) {
+    const Tensor& d = *decay;
+    f32t(d, "decay", false);
+    if (d.dim() == 1) {
+      TORCH_CHECK(d.size(0) == p.H && (p.H == 1 || d.stride(0) == 1), "decay [H]");
+      p.decay_kind = 1;
+    } else if (d.dim() == 2) {
+      col_view(d, "decay");
+      TORCH_CHECK(d.size(0) == T && d.size(1) == p.H, "decay [T, H]");
+      p.decay_kind = 2;
+      p.ldd = (int)d.stride(0);
+    } else {
+      head_view(d, "decay");
+      TORCH_CHECK(d.size(0) == T && d.size(1) == p.H && d.size(2) == p.D, "decay [T, H, D]");
+      p.decay_kind = 3;
+      p.ldd = (int)d.stride(0);
+    }
+    p.decay = d.data_ptr<float>();
+  }
+  if (beta.has_value()) {
+    col_view(*beta, "beta");
+    TORCH_CHECK(beta->size(0) == T && beta->size(1) == p.H, "beta [T, H]");
+    p.beta = beta->data_ptr<float>();
+    p.ldb = (int)beta->stride(0);
+  }
+  p.state = state.data_ptr<float>();
+  p.q_start = q_start.data_ptr<int>();
+  p.q_len = q_len.data_ptr<int>();
+  p.ctx_len = ctx_len.data_ptr<int>();
+  p.state_slot = state_slot.data_ptr<int>();
+  p.out = out.data_ptr<float>();
+  p.q_scale = (float)q_scale;
+  DSSE_CHECK_HIP(dsse_matrix_scan(&p, cur_stream()));
+}
+
+void gated_head_norm(const Tensor& o, const OptTensor& w, const Tensor& gate, double eps, Tensor& out) {
+  f32t(o, "o");
+  col_view(gate, "gate");
+  gpu(out, "out");
+  TORCH_CHECK(o.dim() == 3 && out.dim() == 2, "o [T, H, V], out [T, H V]");
+  const int M = (int)o.size(0), H = (int)o.size(1), V = (int)o.size(2);
+  TORCH_CHECK(gate.size(0) == M && gate.size(1) == (int64_t)H * V && out.size(0) == M && out.size(1) == (int64_t)H * V,
+              "gate and out must be [T, H V]");
+  DSSE_CHECK_HIP(dsse_gated_head_norm(o.data_ptr<float>(), opt_f32(w, "w", V), gate.data_ptr<float>(),
+                                      (int)gate.stride(0), out.data_ptr(), M, H, V, (float)eps, elem(out, "out"),
+                                      cur_stream()));
+}
+
+void rms_mix(const Tensor& ya, const Tensor& wa, const Tensor& yb, const Tensor& wb, double eps, double coef, Tensor& out) {
+  f32t(ya, "ya");
+  f32t(yb, "yb");
+  f32t(out, "out");
+  TORCH_CHECK(ya.dim() == 2 && yb.sizes() == ya.sizes() && out.sizes() == ya.sizes(), "ya, yb, out must be [M, W]");
+  const int M = (int)ya.size(0), W = (int)ya.size(1);
+  f32t(wa, "wa");
+  f32t(wb, "wb");
+  TORCH_CHECK(wa.numel() == W && wb.numel() == W, "gains must be [W]");
+  DSSE_CHECK_HIP(dsse_rms_mix(ya.data_ptr<float>(), wa.data_ptr<float>(), yb.data_ptr<float>(), wb.data_ptr<float>(),
+                              out.data_ptr<float>(), M, W, (float)eps, (float)coef, cur_stream()));
+}
+
+void logit_cap(Tensor& logits, double scale, double cap) {
+  f32t(logits, "logits");
+  DSSE_CHECK_HIP(dsse_logit_cap(logits.data_ptr<float>(), (long long)logits.numel(), (float)scale, (float)cap,
+                                cur_stream()));
+}
+
+}  // namespace
+
+TORCH_LIBRARY_FRAGMENT(dsse, m) {
+  m.def("stream_step(Tensor? y, float mult, Tensor(a!) resid, Tensor? ids, Tensor? embed, Tensor? vec, Tensor? alpha, "
+        "Tensor? w, Tensor? b, Tensor(b!)? xb) -> ()");
+  m.def("gated_act(Tensor gu, Tensor(a!) h, int kind=1) -> ()");
+  m.def("norm_rope_rows(Tensor x, Tensor? norm_w, Tensor positions, Tensor? rope, Tensor(a!) out, Tensor? out_rows, "
+        "int kind, float eps, float scale=1.0) -> ()");
+  m.def("sink_attention(Tensor q, Tensor kcache, Tensor vcache, Tensor block_tables, Tensor q_start, Tensor q_len, "
+        "Tensor ctx_len, Tensor work_seq, Tensor work_tile, Tensor? sink, Tensor? gate, Tensor(a!) out, int window, "
+        "float scale, int qt) -> ()");
+  m.def("gate_math(Tensor(a!) x, int kind, Tensor? p1=None, Tensor? p2=None, float c=1.0) -> ()");
+  m.def("matrix_scan(Tensor q, Tensor k, Tensor v, Tensor? decay, Tensor? beta, Tensor(a!) state, Tensor q_start, "
+        "Tensor q_len, Tensor ctx_len, Tensor state_slot, Tensor(b!) out, float q_scale=1.0) -> ()");
+  m.def("gated_head_norm(Tensor o, Tensor? w, Tensor gate, float eps, Tensor(a!) out) -> ()");
+  m.def("rms_mix(Tensor ya, Tensor wa, Tensor yb, Tensor wb, float eps, float coef, Tensor(a!) out) -> ()");
+  m.def("logit_cap(Tensor(a!) logits, float scale, float cap) -> ()");
+}
+
+TORCH_LIBRARY_IMPL(dsse, CUDA, m) {
+  m.impl("stream_step", &stream_step);
+  m.impl("gated_act", &gated_act);
+  m.impl("norm_rope_rows", &norm_rope_rows);
+  m.impl("sink_attention", &sink_attention);
+  m.impl("gate_math", &gate_math);
+  m.impl("matrix_scan", &matrix_scan);
+  m.impl("gated_head_norm", &gated_head_norm);
+  m.impl("rms_mix", &rms_mix);
+  m.impl("logit_cap", &logit_cap);
+}

@@ -39,16 +39,17 @@ __global__ __launch_bounds__(256) void conv_state_kernel(ConvStateParams p) {
   const T* taps = reinterpret_cast<const T*>(p.taps) + (int64_t)c * K;
   const float bias = p.bias ? (float)reinterpret_cast<const T*>(p.bias)[c] : 0.0f;
   const float ib = p.in_bias ? (float)reinterpret_cast<const T*>(p.in_bias)[c] : 0.0f;  // the input projection's bias
-  const float* in = p.in + (int64_t)row0 * p.C + c;
+  const float* in = p.in + (int64_t)row0 * p.ld_in + c;
   for (int t = t0; t < t1; ++t) {
     float v = bias;
     for (int k = 0; k < K; ++k) {
       const int i = t - Kt + k;
-      const float x = i >= 0 ? in[(int64_t)i * p.C] + ib : (fresh ? 0.0f : tail[(int64_t)(Kt + i) * p.C]);
+      const float x = i >= 0 ? in[(int64_t)i * p.ld_in] + ib : (fresh ? 0.0f : tail[(int64_t)(Kt + i) * p.C]);
       v += (float)taps[k] * x;
     }
+    if (p.act == 1) v = v / (1.0f + expf(-v));
     p.out[(int64_t)(row0 + t) * p.C + c] = v;
-    reinterpret_cast<T*>(p.out_b)[(int64_t)(row0 + t) * p.C + c] = (T)v;
+    if (p.out_b) reinterpret_cast<T*>(p.out_b)[(int64_t)(row0 + t) * p.C + c] = (T)v;
   }
 }
 
@@ -65,10 +66,10 @@ __global__ __launch_bounds__(256) void conv_tail_kernel(ConvStateParams p) {
   const bool fresh = p.ctx_len[seq] - ql == 0;
   float* tail = p.tail + (int64_t)p.state_slot[seq] * Kt * p.C + c;
   const float ib = p.in_bias ? (float)reinterpret_cast<const T*>(p.in_bias)[c] : 0.0f;
-  const float* in = p.in + (int64_t)p.q_start[seq] * p.C + c;
+  const float* in = p.in + (int64_t)p.q_start[seq] * p.ld_in + c;
   for (int j = 0; j < Kt; ++j) {
     const int i = ql - Kt + j;
-    tail[(int64_t)j * p.C] = i >= 0 ? in[(int64_t)i * p.C] + ib : (fresh ? 0.0f : tail[(int64_t)(Kt + i) * p.C]);
+    tail[(int64_t)j * p.C] = i >= 0 ? in[(int64_t)i * p.ld_in] + ib : (fresh ? 0.0f : tail[(int64_t)(Kt + i) * p.C]);
   }
 }
 
