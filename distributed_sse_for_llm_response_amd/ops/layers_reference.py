@@ -115,7 +115,7 @@ def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, 
             continue
         r0, slot = int(q_start[s]), int(state_slot[s])
         fresh = int(ctx_len[s]) - ql == 0
-        prev = torch.zeros(K - 1, inp.shape[1]) if fresh else tail[slot].clone()
+        prev = torch.zeros(K - 1, inp.shape[1]) if fresh or K == 1 else tail[slot].clone()
         seq = torch.cat([prev, inp[r0:r0 + ql].float() + ib])
         y = torch.zeros(ql, inp.shape[1]) if bias is None else bias.float().expand(ql, -1).clone()
         for k in range(K):

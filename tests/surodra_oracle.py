@@ -156,7 +156,7 @@ MIXERS = {"delta": delta_mixer, "parallel": parallel_mixer, "retention": retenti
 
 
 def layer(x, w: dict, i: int, L: dict, cfg: dict):
-    eps, m = float(cfg["norm"]["eps"]), float(cfg["residual_mult"])
+    eps, m = float(cfg["norm"]["eps"]), float(cfg.get("residual_mult", 1.0))
     p = f"l{i}."
     x = x + m * MIXERS[L["type"]](tanh_norm(x, w, p + "norm1"), w, p + "mix.", L["mixer"], eps)
     if L.get("mlp"):
@@ -190,6 +190,6 @@ def forward(cfg: dict, weights: dict, tokens, trace: list | None = None):
         x = layer(x, w, i, cfg["layers"][i], cfg)
         if trace is not None:
             trace.append(x.clone())
-    z = tanh_norm(x, w, "final.norm") @ w["head"].T * float(cfg["logit_scale"])
-    cap = float(cfg["logit_softcap"])
-    return cap * torch.tanh(z / cap)
+    z = tanh_norm(x, w, "final.norm") @ w["head"].T * float(cfg.get("logit_scale", 1.0))
+    cap = cfg.get("logit_softcap")
+    return float(cap) * torch.tanh(z / float(cap)) if cap else z
