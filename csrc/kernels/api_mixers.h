@@ -35,6 +35,7 @@ struct NormRopeParams {
   const float2* rope;    // [rope_len, half] (cos, sin) or null
   void* out;             // rows ldo apart, [nh, D] each; fp32 when out_f32 else bf16
   const int* out_rows;   // [T] or null (row t); negative = skip
+  void* out_t;           // with out_rows: also into transposed pages [pages, nh, D, kBS] (bf16), token permuted, or null
   int T, nh, D, ldx, ldo, half, rope_len, num_out_rows;
   int kind;              // 0 none, 1 RMS over the whole row times norm_w, 2 unit vector per head
   float eps, scale;
@@ -84,6 +85,9 @@ hipError_t dsse_stream_step(const dsse::StreamStepParams* p, hipStream_t st);
 hipError_t dsse_gated_act(const float* gu, int ldg, void* h, int M, int F, int kind, int f32, hipStream_t st);
 hipError_t dsse_norm_rope_rows(const dsse::NormRopeParams* p, hipStream_t st);
 hipError_t dsse_sink_attention(int num_work, const dsse::SinkAttnParams* p, hipStream_t st);
+// MFMA form for prompt portions (bf16, D % 32 == 0, V / 16 in {1..8, 10, 12, 16, 20, 24, 32}): 16-row tiles, values from the
+// transposed pages vt [pages, G, V, kBS] (keys permuted inside a page as the MFMA's k axis wants them)
+hipError_t dsse_sink_flash(int num_work, const dsse::SinkAttnParams* p, const void* vt, hipStream_t st);
 hipError_t dsse_gate_math(float* x, int ld, int M, int N, int kind, const float* p1, const float* p2, float c,
                           hipStream_t st);
 hipError_t dsse_matrix_scan(const dsse::MatrixScanParams* p, hipStream_t st);

@@ -122,7 +122,7 @@ void gated_act(const Tensor& gu, Tensor& h, int64_t kind) {
 }
 
 void norm_rope_rows(const Tensor& x, const OptTensor& norm_w, const Tensor& positions, const OptTensor& rope, Tensor& out,
-                    const OptTensor& out_rows, int64_t kind, double eps, double scale) {
+                    const OptTensor& out_rows, int64_t kind, double eps, double scale, const OptTensor& out_t) {
   head_view(x, "x");
   dsse::NormRopeParams p{};
   p.T = (int)x.size(0), p.nh = (int)x.size(1), p.D = (int)x.size(2);
@@ -153,7 +153,16 @@ void norm_rope_rows(const Tensor& x, const OptTensor& norm_w, const Tensor& posi
     p.out_rows = out_rows->data_ptr<int>();
     p.ldo = p.nh * p.D;
     p.num_out_rows = (int)(out.numel() / p.ldo);
+    if (out_t.has_value()) {  // transposed pages [pages, nh, D, 32] beside the row-major ones
+      gpu(*out_t, "out_t");
+      TORCH_CHECK(out_t->scalar_type() == out.scalar_type() && out_t->dim() == 4 && out_t->size(1) == p.nh &&
+                      out_t->size(2) == p.D && out_t->size(3) == dsse::kBS &&
+                      out_t->size(0) * dsse::kBS == p.num_out_rows,
+                  "out_t must be [pages, heads, width, 32] over the same pages as out");
+      p.out_t = out_t->data_ptr();
+    }
   } else {
+    TORCH_CHECK(!out_t.has_value(), "out_t needs out_rows");
     TORCH_CHECK(out.dim() == 3 && out.sizes() == x.sizes() && (p.D == 1 || out.stride(2) == 1) &&
                     (p.nh == 1 || out.stride(1) == p.D) && out.stride(0) >= (int64_t)p.nh * p.D,
                 "out must be [rows, heads, width] with adjacent heads");
@@ -167,7 +176,7 @@ void norm_rope_rows(const Tensor& x, const OptTensor& norm_w, const Tensor& posi
 void sink_attention(const Tensor& q, const Tensor& kcache, const Tensor& vcache, const Tensor& block_tables,
                     const Tensor& q_start, const Tensor& q_len, const Tensor& ctx_len, const Tensor& work_seq,
                     const Tensor& work_tile, const OptTensor& sink, const OptTensor& gate, Tensor& out, int64_t window,
-                    double scale, int64_t qt) {
+                    double scale, int64_t qt, const OptTensor& vt) {
   f32t(q, "q");
   gpu(kcache, "kcache");
   gpu(vcache, "vcache");
@@ -213,6 +222,16 @@ void sink_attention(const Tensor& q, const Tensor& kcache, const Tensor& vcache,
   p.window = (int)std::min<int64_t>(window, INT_MAX), p.qt = (int)qt;
   p.scale = (float)scale;
   p.f32 = elem(kcache, "kcache");
+  if (vt.has_value()) {  // MFMA form: work_tile counts tiles of 16 rows
+    gpu(*vt, "vt");
+    TORCH_CHECK(kcache.scalar_type() == at::kBFloat16 && vt->scalar_type() == at::kBFloat16, "the MFMA form is bf16");
+    TORCH_CHECK(vt->dim() == 4 && vt->size(0) == vcache.size(0) && vt->size(1) == p.G && vt->size(2) == p.V &&
+                    vt->size(3) == dsse::kBS,
+                "vt must be [pages, G, V, 32]");
+    TORCH_CHECK(qt == 16 && p.D % 32 == 0 && p.V % 16 == 0, "the MFMA form needs qt = 16, D % 32 == 0, V % 16 == 0");
+    DSSE_CHECK_HIP(dsse_sink_flash((int)work_seq.numel(), &p, vt->data_ptr(), cur_stream()));
+    return;
+  }
   DSSE_CHECK_HIP(dsse_sink_attention((int)work_seq.numel(), &p, cur_stream()));
 }
 
@@ -323,10 +342,10 @@ TORCH_LIBRARY_FRAGMENT(dsse, m) {
         "Tensor? w, Tensor? b, Tensor(b!)? xb) -> ()");
   m.def("gated_act(Tensor gu, Tensor(a!) h, int kind=1) -> ()");
   m.def("norm_rope_rows(Tensor x, Tensor? norm_w, Tensor positions, Tensor? rope, Tensor(a!) out, Tensor? out_rows, "
-        "int kind, float eps, float scale=1.0) -> ()");
+        "int kind, float eps, float scale=1.0, Tensor(b!)? out_t=None) -> ()");
   m.def("sink_attention(Tensor q, Tensor kcache, Tensor vcache, Tensor block_tables, Tensor q_start, Tensor q_len, "
         "Tensor ctx_len, Tensor work_seq, Tensor work_tile, Tensor? sink, Tensor? gate, Tensor(a!) out, int window, "
-        "float scale, int qt) -> ()");
+        "float scale, int qt, Tensor? vt=None) -> ()");
   m.def("gate_math(Tensor(a!) x, int kind, Tensor? p1=None, Tensor? p2=None, float c=1.0) -> ()");
   m.def("matrix_scan(Tensor q, Tensor k, Tensor v, Tensor? decay, Tensor? beta, Tensor(a!) state, Tensor q_start, "
         "Tensor q_len, Tensor ctx_len, Tensor state_slot, Tensor(b!) out, float q_scale=1.0) -> ()");

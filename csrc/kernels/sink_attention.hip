@@ -8,7 +8,7 @@
 // "nothing".  Scores, the running maximum, the weights and the output sums are fp32 in both element types; queries
 // arrive in fp32 (normed and rotated), keys and values are read from their pages in the cache's element type.
 //
-// Row kernel: a workgroup serves `qt` query rows of one head; for each row its four waves split the keys in chunks of
+// Row kernel (any sizes, both element types; every decode step): a workgroup serves `qt` query rows of one head; for each row its four waves split the keys in chunks of
 // 64 (one key per lane for the scores, then one output coordinate per lane and 64 broadcast weights for the values),
 // keep their own running (max, sum, output) and are merged through LDS.  A decode row and a prompt row take the same
 // path, so a position's result does not depend on how the prompt was cut.
@@ -130,8 +130,170 @@ __global__ __launch_bounds__(256) void sink_attention_kernel(SinkAttnParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// MFMA form for prompt portions (bf16; D % 32 == 0, V % 16 == 0): one wave per (16 query rows, head), 32 keys (one
+// page) per step, a workgroup = up to four heads of the same rows (heads of one key/value group read the same pages,
+// which then come from the CU's L1).
+//
+//   S^T[key, row] = K[key, :] . Q[row, :]    A = the page's key rows straight from global memory (16 B per lane),
+//                                             B = the 16 rows' query vectors staged in LDS as bf16
+//   online softmax per row in fp32 (a row's 32 scores sit in 8 registers of its 4 lanes)
+//   O^T[dim, row] += V^T[dim, key] . P^T[key, row]
+//                                             A = the TRANSPOSED value page vt[page][G][V][32 keys] (16 B per lane),
+//                                             B = the weights exactly as the score accumulators hold them
+//
+// Which key an (lane group g, element j) pair of the k axis stands for only has to agree between A and B: the scores of
+// lane group g are keys 4g..4g+3 of both 16-key halves, so the transposed page stores key k at position
+// 8 ((k & 15) >> 2) + 4 (k >> 4) + (k & 3).  The sink enters once, when the row is finished: it only enlarges the
+// denominator.
+template <int NT>  // V / 16 value tiles
+__global__ __launch_bounds__(256) void sink_flash_kernel(SinkAttnParams p, const bf16* __restrict__ vt, int head_tiles) {
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  const int D = p.D, V = p.V;
+  const int ldq = D + 8;  // bf16 elements per LDS row (16 B of padding)
+  const int wave = threadIdx.x >> 6;
+  const int h = blockIdx.y * (blockDim.x >> 6) + wave;
+  bf16* qs = reinterpret_cast<bf16*>(smem_raw) + wave * 16 * ldq;
+  const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+  const int seq = p.work_seq[blockIdx.x], tile = p.work_tile[blockIdx.x];
+  const int ql = p.q_len[seq];
+  if (tile * 16 >= ql) return;
+  const bool h_ok = h < head_tiles;
+  const int hh = h_ok ? h : 0;
+  const int kvh = hh / (p.H / p.G);
+  const int q0 = p.q_start[seq], pos0 = p.ctx_len[seq] - ql;
+  const int c_off = tile * 16 + r;
+  const bool c_ok = c_off < ql && h_ok;
+  const int c_pos = c_ok ? pos0 + c_off : -1;
+  const int64_t c_row = q0 + (c_off < ql ? c_off : 0);
+  {
+    const float* qa = p.q + (c_row * p.H + hh) * D;
+    for (int d = 8 * g; d < D; d += 32) {
+      const f32x4 lo4 = c_ok ? *reinterpret_cast<const f32x4*>(qa + d) : f32x4{0.f, 0.f, 0.f, 0.f};
+      const f32x4 hi4 = c_ok ? *reinterpret_cast<const f32x4*>(qa + d + 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+      bf16x8 v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = (bf16)lo4[j], v[4 + j] = (bf16)hi4[j];
+      *reinterpret_cast<bf16x8*>(qs + r * ldq + d) = v;
+    }
+  }
+  __syncthreads();
+  if (!h_ok) return;
+  const int last_off = tile * 16 + 15 < ql ? tile * 16 + 15 : ql - 1;
+  const int hi = pos0 + last_off;
+  int lo = pos0 + tile * 16 - p.window + 1;
+  lo = lo > 0 ? lo : 0;
+  const int* bt = p.block_tables + (int64_t)seq * p.max_blocks;
+  const bf16* kc = reinterpret_cast<const bf16*>(p.k);
+  f32x4 O[NT];
+#pragma unroll
+  for (int n = 0; n < NT; ++n) O[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int nks = D / 32;
+  for (int pg = lo / kBS; pg <= hi / kBS; ++pg) {
+    int blk = bt[pg];
+    blk = (unsigned)blk < (unsigned)p.num_blocks ? blk : 0;
+    const bf16* krow0 = kc + (((int64_t)blk * kBS + r) * p.G + kvh) * D + 8 * g;  // key r of the page's first half
+    const bf16* krow1 = krow0 + (int64_t)16 * p.G * D;                              // key 16 + r
+    const bf16* vrow = vt + (((int64_t)blk * p.G + kvh) * V + r) * kBS + 8 * g;   // dim r of value tile 0
+    bf16x8 vf[NT];
+#pragma unroll
+    for (int n = 0; n < NT; ++n) vf[n] = ld_global<bf16x8>(vrow + (int64_t)n * 16 * kBS);
+    f32x4 s0 = f32x4{0.f, 0.f, 0.f, 0.f}, s1 = s0;
+    for (int sb = 0; sb < nks; sb += 4) {  // four k-steps of key loads are requested before the first MFMA needs one
+      bf16x8 ka[4], kb[4], qb[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int s = sb + u < nks ? sb + u : nks - 1;
+        ka[u] = ld_global<bf16x8>(krow0 + 32 * s);
+        kb[u] = ld_global<bf16x8>(krow1 + 32 * s);
+        qb[u] = *reinterpret_cast<const bf16x8*>(qs + r * ldq + 32 * s + 8 * g);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (sb + u < nks) {
+          s0 = mfma16x16x32(ka[u], qb[u], s0);
+          s1 = mfma16x16x32(kb[u], qb[u], s1);
+        }
+      }
+    }
+    float sv[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int key = pg * kBS + (i < 4 ? 4 * g + i : 16 + 4 * g + (i - 4));
+      const bool seen = c_ok && key <= c_pos && c_pos - key < p.window;
+      sv[i] = seen ? (i < 4 ? s0[i] : s1[i - 4]) * p.scale : -INFINITY;
+      mx = fmaxf(mx, sv[i]);
+    }
+    mx = rows4_max(mx);
+    const float mn = fmaxf(m, mx);
+    const float corr = mn == -INFINITY ? 1.0f : expf(m - mn);
+    bf16x8 pf;
+    float ps = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float e = sv[i] == -INFINITY ? 0.0f : expf(sv[i] - mn);
+      ps += e;
+      pf[i] = (bf16)e;
+    }
+    l = l * corr + rows4_sum(ps);
+    m = mn;
+#pragma unroll
+    for (int n = 0; n < NT; ++n) {
+      f32x4 o = O[n];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] *= corr;
+      O[n] = mfma16x16x32(vf[n], pf, o);
+    }
+  }
+  if (c_ok) {
+    float den = l, f = 1.0f;
+    if (p.sink) {  // the sink joins the denominator under the common maximum
+      const float sk = p.sink[h];
+      const float mm = fmaxf(m, sk);
+      f = expf(m - mm);
+      den = l * f + expf(sk - mm);
+    }
+    float inv = den > 0.f ? f / den : 0.0f;
+    if (p.gate) inv *= 1.0f / (1.0f + expf(-p.gate[c_row * p.ldg + h]));
+    bf16* out = reinterpret_cast<bf16*>(p.out) + (c_row * p.H + h) * V;
+#pragma unroll
+    for (int n = 0; n < NT; ++n) {
+      bf16x4 v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = (bf16)(O[n][i] * inv);
+      *reinterpret_cast<bf16x4*>(out + 16 * n + 4 * g) = v;
+    }
+  }
+}
+
+template <int NT>
+void launch_flash(int num_work, const SinkAttnParams& p, const bf16* vt, hipStream_t st) {
+  const int wy = p.H < 4 ? p.H : 4;
+  const size_t lds = wy * 16 * (size_t)(p.D + 8) * sizeof(bf16);
+  dim3 grid(num_work, (p.H + wy - 1) / wy), block(64 * wy);
+  hipLaunchKernelGGL(sink_flash_kernel<NT>, grid, block, lds, st, p, vt, p.H);
+}
+
 }  // namespace
 }  // namespace dsse
+
+// work_tile counts tiles of 16 rows; vt: transposed value pages [pages, G, V, kBS], keys permuted inside a page
+extern "C" hipError_t dsse_sink_flash(int num_work, const dsse::SinkAttnParams* p, const void* vt, hipStream_t st) {
+  if (num_work <= 0 || p->H <= 0) return hipSuccess;
+  if (p->f32 || p->D % 32 || p->V % 16 || p->V > 512 || p->D > 512 || p->H % p->G) return hipErrorInvalidValue;
+  const bf16* v = reinterpret_cast<const bf16*>(vt);
+  switch (p->V / 16) {
+#define DSSE_FLASH_CASE(n) case n: dsse::launch_flash<n>(num_work, *p, v, st); break;
+    DSSE_FLASH_CASE(1) DSSE_FLASH_CASE(2) DSSE_FLASH_CASE(3) DSSE_FLASH_CASE(4) DSSE_FLASH_CASE(5) DSSE_FLASH_CASE(6)
+    DSSE_FLASH_CASE(7) DSSE_FLASH_CASE(8) DSSE_FLASH_CASE(10) DSSE_FLASH_CASE(12) DSSE_FLASH_CASE(16)
+    DSSE_FLASH_CASE(20) DSSE_FLASH_CASE(24) DSSE_FLASH_CASE(32)
+#undef DSSE_FLASH_CASE
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
 
 extern "C" hipError_t dsse_sink_attention(int num_work, const dsse::SinkAttnParams* p, hipStream_t st) {
   if (num_work <= 0 || p->H <= 0) return hipSuccess;

@@ -119,6 +119,11 @@ __global__ __launch_bounds__(256) void norm_rope_rows_kernel(NormRopeParams p) {
           v = lo ? v * c.x - o * c.y : v * c.x + o * c.y;
         }
         out[h * p.D + i] = (OutT)(v * p.scale);
+        if (p.out_t) {  // the same number once more where the MFMA attention's value operand wants it
+          const int page = orow / kBS, off = orow % kBS;
+          const int at = ((off & 15) >> 2) * 8 + ((off >> 4) & 1) * 4 + (off & 3);
+          reinterpret_cast<OutT*>(p.out_t)[(((int64_t)page * p.nh + h) * p.D + i) * kBS + at] = (OutT)(v * p.scale);
+        }
       }
     __syncthreads();  // the strip is read before the next head overwrites it
   }

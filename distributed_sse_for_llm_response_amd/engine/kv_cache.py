@@ -108,10 +108,15 @@ class PagedKVCache:
     block tables and allocator as the other caches (a page id means the same page in every run).  ``shapes`` maps a
     run's key -> (G, D, V); a layer that runs several times (a looped span) has one entry per run."""
 
-    def __init__(self, shapes: dict, num_blocks: int, device, dtype=torch.bfloat16):
+    def __init__(self, shapes: dict, num_blocks: int, device, dtype=torch.bfloat16, transposed=()):
         self.num_blocks = num_blocks
         self.k = {r: torch.zeros(num_blocks, PAGE, g, d, device=device, dtype=dtype) for r, (g, d, _) in shapes.items()}
         self.v = {r: torch.zeros(num_blocks, PAGE, g, v, device=device, dtype=dtype) for r, (g, _, v) in shapes.items()}
+        # runs on the MFMA attention form also keep the values in transposed pages [blocks, G, V, PAGE] (tokens
+        # permuted inside a page, ops/layers_reference.py vt_position): the prompt kernel's value operand is then one
+        # 16-byte load per lane; decode steps read the row-major pages
+        self.vt = {r: torch.zeros(num_blocks, shapes[r][0], shapes[r][2], PAGE, device=device, dtype=dtype)
+                   for r in transposed}
 
     @staticmethod
     def bytes_per_block(shapes: dict, elem_bytes: int = 2) -> int:

@@ -39,6 +39,7 @@ from .weights import LayeredWeights
 
 ATTN_ROWS_TILE = 4    # query rows per work item of the row-wise attention kernel (prompt portions)
 FLASH_DECODE_WAVES = 512  # waves a decode attention launch aims for (two per CU)
+SINK_ROWS_TILE = 16   # query rows per work item of the sink attention's MFMA form (one head per wave)
 FLASH_ROWS_TILE = 4   # query rows per work item of the MFMA attention form, x 4 heads = 16 columns: a page of keys is
                       # read once for four heads (16 rows x 1 head re-read it per head: 2-3x the time at 16 heads)
 
@@ -103,7 +104,8 @@ class LayeredRunner(RunnerBase):
             rot = m.left.rot if L.kind == "parallel" else getattr(m, "rot", None)
             if rot is not None and rot.dims > 0 and rot not in self._rope:
                 self._rope[rot] = rot.table(self.max_model_len + 1, dev)
-        self.kv = PagedKVCache(kv, self.num_blocks, dev, self.dtype)
+        flash = [r for r, (_, d, v) in kv.items() if ops.sink_flash_ok(self.dtype, d, v)]
+        self.kv = PagedKVCache(kv, self.num_blocks, dev, self.dtype, transposed=flash)
         self.state = MatrixStateCache(st, self.max_batch, dev)
 
     # ------------------------------------------------------------------ buffers
@@ -383,11 +385,16 @@ class LayeredRunner(RunnerBase):
         qa = d["qa"][:M * H * D].view(M, H, D)
         ops.norm_rope_rows(self._cols(big, 0, H, D), Lw.q_norm, pos, rope, qa, None, 1, self.cfg.eps, 1.0)
         ops.norm_rope_rows(self._cols(big, H * D, G, D), Lw.k_norm, pos, rope, self.kv.k[ri], slots, 1, self.cfg.eps, 1.0)
-        ops.norm_rope_rows(self._cols(big, (H + G) * D, G, V), None, pos, None, self.kv.v[ri], slots, 0, 0.0, 1.0)
+        vt = self.kv.vt.get(ri)
+        ops.norm_rope_rows(self._cols(big, (H + G) * D, G, V), None, pos, None, self.kv.v[ri], slots, 0, 0.0, 1.0, vt)
         ao = d["ao"][:M * H * V].view(M, H, V)
         for g in groups:
-            ops.sink_attention(qa, self.kv.k[ri], self.kv.v[ri], g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"], g["wt"],
-                               Lw.sink, small[:, :H], ao, a.window, a.scale, g["qt"])
+            if vt is not None and g["qt"] > 1:  # prompt portions on the MFMA form: tiles of 16 rows
+                ops.sink_attention(qa, self.kv.k[ri], self.kv.v[ri], g["bt"], g["qs"], g["ql"], g["ctx"], g["hs"],
+                                   g["ht"], Lw.sink, small[:, :H], ao, a.window, a.scale, SINK_ROWS_TILE, vt)
+            else:
+                ops.sink_attention(qa, self.kv.k[ri], self.kv.v[ri], g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"],
+                                   g["wt"], Lw.sink, small[:, :H], ao, a.window, a.scale, g["qt"])
         self._lin(ao.view(M, H * V), Lw.lo, Lw.lo_t, d["y"])
         # right: gated linear attention, decay per key channel from the low-rank projection (fp32 throughout)
         z = d["z"][:M * Hr * Dr].view(M, Hr * Dr)
@@ -473,7 +480,7 @@ class LayeredRunner(RunnerBase):
         """Packed metadata of prompt portions whose rows start at `row0`: one pinned upload.  Returns (T, q_start
         list, device dict: ids / pos / slots per row, qs / ql / ctx / ss per sequence, ws / wt work items, bt)."""
         n = len(seqs)
-        ids_l, pos_l, slots_l, qs, ql, ctx, ss, ws, wt, fs, ft = [], [], [], [], [], [], [], [], [], [], []
+        ids_l, pos_l, slots_l, qs, ql, ctx, ss, ws, wt, fs, ft, hs, ht = [], [], [], [], [], [], [], [], [], [], [], [], []
         bt = torch.zeros(n, self.max_blocks, dtype=torch.int32)
         row = 0
         for i, s in enumerate(seqs):
@@ -494,16 +501,20 @@ class LayeredRunner(RunnerBase):
             nf = math.ceil(m / FLASH_ROWS_TILE)
             fs += [i] * nf
             ft += list(range(nf))
+            nh = math.ceil(m / SINK_ROWS_TILE)
+            hs += [i] * nh
+            ht += list(range(nh))
             row += m
         T = row
-        meta = torch.from_numpy(np.concatenate(ids_l + pos_l + slots_l + [np.asarray(qs + ql + ctx + ss + ws + wt + fs + ft,
+        meta = torch.from_numpy(np.concatenate(ids_l + pos_l + slots_l + [np.asarray(qs + ql + ctx + ss + ws + wt + fs + ft + hs + ht,
                                                                                      dtype=np.int64)]).astype(np.int32))
         if self.device.type == "cuda":
             meta = meta.pin_memory().to(self.device, non_blocking=True)
             bt = bt.pin_memory().to(self.device, non_blocking=True)
         d, o = {}, 0
         for name, k in (("ids", T), ("pos", T), ("slots", T), ("qs", n), ("ql", n), ("ctx", n), ("ss", n),
-                        ("ws", len(ws)), ("wt", len(ws)), ("fs", len(fs)), ("ft", len(fs))):
+                        ("ws", len(ws)), ("wt", len(ws)), ("fs", len(fs)), ("ft", len(fs)), ("hs", len(hs)),
+                        ("ht", len(hs))):
             d[name], o = meta[o:o + k], o + k
         d["bt"] = bt
         d["qt"] = ATTN_ROWS_TILE

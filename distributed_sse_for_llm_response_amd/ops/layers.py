@@ -157,27 +157,37 @@ def gated_act(gu, h, kind: int = 1):
         lref.gated_act(gu, h, kind)
 
 
-def norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind: int, eps: float, scale: float = 1.0):
+def norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind: int, eps: float, scale: float = 1.0, out_t=None):
     """Rows x [T, heads, D] (fp32, may be a column slice of a wider buffer) -> out rows out_rows[t] (or t) in out's
     type: an optional norm (1: RMS over the whole row times norm_w; 2: unit vector per head), the rotate-half rotation
     of the leading 2 * rope.shape[1] coordinates (rope [positions, dims / 2, 2] or None), times scale.  With out_rows =
-    cache rows this writes keys or values straight into their pages."""
+    cache rows this writes keys or values straight into their pages [pages, 32, heads, D]; out_t (optional,
+    [pages, heads, D, 32]) receives them once more in transposed pages (the MFMA attention's value operand)."""
     if _hip(x):
-        torch.ops.dsse.norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind, eps, scale)
+        torch.ops.dsse.norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind, eps, scale, out_t)
     else:
-        lref.norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind, eps, scale)
+        lref.norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind, eps, scale, out_t)
+
+
+SINK_FLASH_TILES = (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16, 20, 24, 32)  # value widths / 16 the MFMA form is built for
+
+
+def sink_flash_ok(dtype, dim: int, vdim: int) -> bool:
+    """Shapes the MFMA form of sink_attention covers (prompt portions; everything else takes the row kernel)."""
+    return dtype == torch.bfloat16 and dim % 32 == 0 and dim <= 512 and vdim % 16 == 0 and vdim // 16 in SINK_FLASH_TILES
 
 
 def sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile, sink, gate, out,
-                   window: int, scale: float, qt: int):
+                   window: int, scale: float, qt: int, vt=None):
     """Causal softmax attention of q [T, H, D] over paged keys [pages, 32, G, D] and values [pages, 32, G, V] (grouped
     heads), scores and weights in fp32; sink [H] adds exp(sink) to each head's denominator, gate [T, H] multiplies the
-    head's output by its sigmoid.  `qt` query rows per work item (work_seq, work_tile)."""
+    head's output by its sigmoid.  `qt` query rows per work item (work_seq, work_tile).  With vt (transposed value
+    pages [pages, G, V, 32], sink_flash_ok shapes, qt = 16): the MFMA form for prompt portions."""
     if _hip(q):
         torch.ops.dsse.sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile,
-                                      sink, gate, out, window, scale, qt)
+                                      sink, gate, out, window, scale, qt, vt)
     else:
-        lref.sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, sink, gate, out, window, scale)
+        lref.sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, sink, gate, out, window, scale, vt)
 
 
 def gate_math(x, kind: int, p1=None, p2=None, c: float = 1.0):

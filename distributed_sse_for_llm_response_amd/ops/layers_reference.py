@@ -242,7 +242,7 @@ def rotate_half_rows(v, cs, dims):
     return out
 
 
-def norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind, eps, scale):
+def norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind, eps, scale, out_t=None):
     """x [T, heads, D] fp32 -> out rows (out_rows[t], or t) as [heads, D] in out's type.  norm_kind 1: RMS norm over
     the whole row (all heads at once) times norm_w [heads * D]; 2: every head divided by sqrt(sum of squares + eps);
     then the rotate-half rotation of the leading 2 * rope.shape[1] coordinates at positions[t]; then times scale.
@@ -265,12 +265,15 @@ def norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind, eps, sc
         r = out_rows[:T].long()
         ok = (r >= 0) & (r < flat_out.shape[0])
         flat_out[r[ok]] = v[ok]
+        if out_t is not None:  # [pages, heads, D, PAGE], the token at vt_position(offset)
+            good = r[ok]
+            out_t[good // PAGE, :, :, vt_position(good % PAGE)] = v[ok]
 
 
-def sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, sink, gate, out, window, scale):
+def sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, sink, gate, out, window, scale, vt=None):
     """Softmax attention over paged keys [pages, PAGE, G, D] and values [pages, PAGE, G, V] with grouped heads; the
     denominator also holds exp(sink[h]) when sink is given; the head's output is multiplied by sigmoid(gate[row, h])
-    when gate is given."""
+    when gate is given.  With vt the values come from the transposed pages [pages, G, V, PAGE]."""
     H = q.shape[1]
     G = kcache.shape[2]
     kf = kcache.view(-1, G, kcache.shape[3]).float()
@@ -287,6 +290,8 @@ def sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, sin
             j = torch.arange(max(0, pos - window + 1), pos + 1)
             rows = bt[j // PAGE] * PAGE + j % PAGE
             k, v = kf[rows][:, grp], vf[rows][:, grp]                       # [keys, H, D], [keys, H, V]
+            if vt is not None:  # the same numbers from the transposed pages, so a wrong place shows
+                v = vt[rows // PAGE, :, :, vt_position(rows % PAGE)].float()[:, grp]
             sc = torch.einsum("hd,jhd->hj", q[r0 + i].float(), k) * scale
             mx = sc.max(-1, keepdim=True).values
             if sink is not None:

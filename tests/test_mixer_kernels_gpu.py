@@ -153,6 +153,52 @@ def test_sink_attention(dtype, H, G, D, V, window):
         close(o, o_ref, 1e-5 if dtype == torch.float32 else 1e-2)
 
 
+@pytest.mark.parametrize("H,G,D,V,window", [(4, 2, 64, 64, 10 ** 9), (6, 1, 32, 16, 37), (5, 5, 128, 112, 10 ** 9),
+                                            (8, 2, 96, 320, 100)])
+def test_sink_attention_mfma_form(H, G, D, V, window):
+    """Prompt portions on the MFMA form (values from the transposed pages) against the reference, which reads the same
+    transposed pages: tiles that start and end inside pages, a first token, a portion deep into a long context."""
+    g = torch.Generator().manual_seed(8)
+    ctx, ql = [300, 1, 70, 45], [40, 1, 70, 2]
+    bt, pages = _pages(4, ctx, g)
+    T = sum(ql)
+    q = torch.randn(T, H, D, generator=g)
+    kc = torch.randn(pages, PAGE, G, D, generator=g).to(torch.bfloat16)
+    vc = torch.randn(pages, PAGE, G, V, generator=g).to(torch.bfloat16)
+    off = torch.arange(PAGE)
+    vt = torch.zeros(pages, G, V, PAGE, dtype=torch.bfloat16)
+    vt[:, :, :, lref.vt_position(off)] = vc.permute(0, 2, 3, 1)
+    sink, gate = torch.randn(H, generator=g), torch.randn(T, H, generator=g)
+    qs = i32([0, 40, 41, 111])
+    hs = [s for s, n in enumerate(ql) for _ in range(math.ceil(n / 16))]
+    ht = [t for n in ql for t in range(math.ceil(n / 16))]
+    for use in (True, False):
+        o_ref = torch.zeros(T, H, V, dtype=torch.bfloat16)
+        lref.sink_attention(q, kc, torch.zeros_like(vc), bt, qs, i32(ql), i32(ctx), sink if use else None,
+                            gate if use else None, o_ref, window, 0.2, vt)
+        c = lambda t: t.to(dev())  # noqa: E731
+        o = torch.zeros(T, H, V, dtype=torch.bfloat16, device=dev())
+        ops.sink_attention(c(q), c(kc), c(vc), c(bt), c(qs), c(i32(ql)), c(i32(ctx)), c(i32(hs)), c(i32(ht)),
+                           c(sink) if use else None, c(gate) if use else None, o, window, 0.2, 16, c(vt))
+        close(o, o_ref, 2e-2)
+
+
+def test_transposed_value_pages_written_with_the_rows():
+    g = torch.Generator().manual_seed(9)
+    T, G, V = 40, 2, 48
+    x = torch.randn(T, G, V, generator=g)
+    rows = torch.randperm(3 * PAGE, generator=g)[:T].to(torch.int32)
+    rows[5] = -1
+    ref, ref_t = torch.zeros(3, PAGE, G, V, dtype=torch.bfloat16), torch.zeros(3, G, V, PAGE, dtype=torch.bfloat16)
+    lref.norm_rope_rows(x, None, rows, None, ref, rows, 0, 0.0, 1.0, ref_t)
+    out, out_t = ref.clone().zero_().to(dev()), ref_t.clone().zero_().to(dev())
+    ops.norm_rope_rows(x.to(dev()), None, rows.to(dev()), None, out, rows.to(dev()), 0, 0.0, 1.0, out_t)
+    assert torch.equal(out.cpu(), ref) and torch.equal(out_t.cpu(), ref_t)
+    flat = ref.view(-1, G, V)
+    for r in (0, 17, 95):   # the transposed page holds row r's numbers at vt_position(r % 32)
+        assert torch.equal(ref_t[r // PAGE, :, :, int(lref.vt_position(torch.tensor(r % PAGE)))], flat[r])
+
+
 @pytest.mark.parametrize("H,G,D,V", [(4, 2, 32, 32), (2, 2, 48, 100), (3, 1, 128, 64), (1, 1, 300, 70), (2, 1, 8, 5)])
 @pytest.mark.parametrize("mode", ["delta", "channel", "fixed", "plain"])
 def test_matrix_scan(H, G, D, V, mode):
