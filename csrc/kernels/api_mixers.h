@@ -87,7 +87,8 @@ hipError_t dsse_norm_rope_rows(const dsse::NormRopeParams* p, hipStream_t st);
 hipError_t dsse_sink_attention(int num_work, const dsse::SinkAttnParams* p, hipStream_t st);
 // MFMA form for prompt portions (bf16, D % 32 == 0, V / 16 in {1..8, 10, 12, 16, 20, 24, 32}): 16-row tiles, values from the
 // transposed pages vt [pages, G, V, kBS] (keys permuted inside a page as the MFMA's k axis wants them)
-hipError_t dsse_sink_flash(int num_work, const dsse::SinkAttnParams* p, const void* vt, hipStream_t st);
+// split (V <= 128): the four waves of a workgroup share one (tile, head) and split its pages -- decode steps
+hipError_t dsse_sink_flash(int num_work, const dsse::SinkAttnParams* p, const void* vt, int split, hipStream_t st);
 hipError_t dsse_gate_math(float* x, int ld, int M, int N, int kind, const float* p1, const float* p2, float c,
                           hipStream_t st);
 hipError_t dsse_matrix_scan(const dsse::MatrixScanParams* p, hipStream_t st);

@@ -176,7 +176,7 @@ void norm_rope_rows(const Tensor& x, const OptTensor& norm_w, const Tensor& posi
 void sink_attention(const Tensor& q, const Tensor& kcache, const Tensor& vcache, const Tensor& block_tables,
                     const Tensor& q_start, const Tensor& q_len, const Tensor& ctx_len, const Tensor& work_seq,
                     const Tensor& work_tile, const OptTensor& sink, const OptTensor& gate, Tensor& out, int64_t window,
-                    double scale, int64_t qt, const OptTensor& vt) {
+                    double scale, int64_t qt, const OptTensor& vt, bool split) {
   f32t(q, "q");
   gpu(kcache, "kcache");
   gpu(vcache, "vcache");
@@ -229,7 +229,8 @@ void sink_attention(const Tensor& q, const Tensor& kcache, const Tensor& vcache,
                     vt->size(3) == dsse::kBS,
                 "vt must be [pages, G, V, 32]");
     TORCH_CHECK(qt == 16 && p.D % 32 == 0 && p.V % 16 == 0, "the MFMA form needs qt = 16, D % 32 == 0, V % 16 == 0");
-    DSSE_CHECK_HIP(dsse_sink_flash((int)work_seq.numel(), &p, vt->data_ptr(), cur_stream()));
+    TORCH_CHECK(!split || p.V <= 128, "the key split of the MFMA form needs V <= 128");
+    DSSE_CHECK_HIP(dsse_sink_flash((int)work_seq.numel(), &p, vt->data_ptr(), split ? 1 : 0, cur_stream()));
     return;
   }
   DSSE_CHECK_HIP(dsse_sink_attention((int)work_seq.numel(), &p, cur_stream()));
@@ -345,7 +346,7 @@ TORCH_LIBRARY_FRAGMENT(dsse, m) {
         "int kind, float eps, float scale=1.0, Tensor(b!)? out_t=None) -> ()");
   m.def("sink_attention(Tensor q, Tensor kcache, Tensor vcache, Tensor block_tables, Tensor q_start, Tensor q_len, "
         "Tensor ctx_len, Tensor work_seq, Tensor work_tile, Tensor? sink, Tensor? gate, Tensor(a!) out, int window, "
-        "float scale, int qt, Tensor? vt=None) -> ()");
+        "float scale, int qt, Tensor? vt=None, bool split=False) -> ()");
   m.def("gate_math(Tensor(a!) x, int kind, Tensor? p1=None, Tensor? p2=None, float c=1.0) -> ()");
   m.def("matrix_scan(Tensor q, Tensor k, Tensor v, Tensor? decay, Tensor? beta, Tensor(a!) state, Tensor q_start, "
         "Tensor q_len, Tensor ctx_len, Tensor state_slot, Tensor(b!) out, float q_scale=1.0) -> ()");

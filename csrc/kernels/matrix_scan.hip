@@ -8,38 +8,50 @@
 //     S = S + k u^T
 //     o = S^T (q_scale q)           the read-out sees the current token's write
 //
-// Column j of S evolves independently of the other columns, so the work is laid out by columns: a workgroup owns 64
-// columns of one (sequence, head); wave r of it holds rows [r DPT, (r + 1) DPT) of those columns in registers (one
-// column per lane), and the dot products over D are finished through LDS.
+// Column j of S evolves independently of the other columns, so the work is laid out by columns: a workgroup owns 16
+// columns of one (sequence, head).  Lane (c, dg) of wave r holds DPT rows of column c -- rows (4 r + dg) DPT + i -- in
+// registers, so a dot product over D is DPT FMAs per lane, a sum over the wave's four 16-lane rows (two row swaps, no
+// LDS) and a short sum over the waves through LDS.  A small DPT spreads one head's state over many waves: what bounds a
+// prompt portion is the dependent chain per token, and it is shortest when every lane holds few rows.
 //
 // Tokens are taken in blocks of TB.  A block's k, q (and per-channel decays) are staged in LDS by the whole workgroup
-// with coalesced loads, and the NEXT block is already in flight (in registers) while the current one is walked, so the
-// dependent chain per token is LDS reads and FMAs, not a trip to memory.  The read-out's partial sums of a whole block
-// are reduced at the block's end; only the delta rule needs a workgroup barrier per token (its S^T k sum crosses the
-// waves).  A decode step is one block of one token: one pass over the state (read, update, write, coalesced along V).
-// A sequence whose step starts at position 0 starts from S = 0; nothing is cleared when a slot changes hands.
+// with coalesced loads, and the NEXT block is already in flight (in registers) while the current one is walked.  The
+// read-out's partial sums of a whole block are reduced at the block's end, and a full block is walked without
+// branches, so without the delta rule the tokens of a block overlap (only S itself chains them); the delta rule needs
+// one workgroup barrier per token (its S^T k sum crosses the waves).  A decode step is one block of one token: one pass
+// over the state (read, update, write).  A sequence whose step starts at position 0 starts from S = 0; nothing is
+// cleared when a slot changes hands.
 #include "api_mixers.h"
 
 namespace dsse {
 namespace {
 
-constexpr int kScanCols = 64;
+constexpr int kScanCols = 16;
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding global load, which
+// would land the next block's prefetch at each barrier; here those loads stay in flight until stage() uses them (the
+// compiler's own vmcnt wait at the first use of their registers).
+DEV void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 template <int DPT, int TB, bool DELTA>
-__global__ void matrix_scan_kernel(MatrixScanParams p, int R) {
-  constexpr int E = TB * DPT / 64;  // staged elements of k (and q, a) per thread and block: TB * Dp / (64 R)
-  extern __shared__ float lds[];
+__global__ __launch_bounds__(1024) void matrix_scan_kernel(MatrixScanParams p, int R) {
+  constexpr int RW = 4 * DPT;        // rows of S per wave
+  constexpr int E = TB * RW / 64;    // staged elements of k (and q, a) per thread and block: TB * Dp / (64 R)
+  static_assert(E >= 1 && E * 64 == TB * RW, "a block's staging divides evenly over the workgroup");
+  extern __shared__ __align__(16) float lds[];
   const int seq = blockIdx.z, h = blockIdx.y;
   const int ql = p.q_len[seq];
   if (ql <= 0) return;
   const int tid = threadIdx.x, lane = tid & 63, r = tid >> 6;
+  const int c = lane & 15, dg = lane >> 4;
   const int nthreads = R * 64;
-  const int j = blockIdx.x * kScanCols + lane;
+  const int j = blockIdx.x * kScanCols + c;
   const bool col_on = j < p.V;
   const int g = h / (p.H / p.G);
-  const int D = p.D, Dp = R * DPT;
+  const int D = p.D, Dp = R * RW;
+  const int d0 = (4 * r + dg) * DPT;  // this lane's first row
   const bool chan = p.decay_kind == 3;
-  // LDS: k[2][TB][Dp] | q[2][TB][Dp] | (a[2][TB][Dp]) | sc[2][2][TB] (beta, scalar decay) | part[2][R][64] | opart[TB][R][64]
+  // LDS: k[2][TB][Dp] | q[2][TB][Dp] | (a[2][TB][Dp]) | sc[2][2][TB] (beta, scalar decay) | part[2][R][16] | opart[TB][R][16]
   float* ks = lds;
   float* qs = ks + 2 * TB * Dp;
   float* as = qs + 2 * TB * Dp;
@@ -51,14 +63,10 @@ __global__ void matrix_scan_kernel(MatrixScanParams p, int R) {
   float* st = p.state + (((int64_t)p.state_slot[seq] * p.H + h) * D) * p.V + j;
   float S[DPT];
 #pragma unroll
-  for (int i = 0; i < DPT; ++i) {
-    const int d = r * DPT + i;
-    S[i] = (!fresh && col_on && d < D) ? st[(int64_t)d * p.V] : 0.0f;
-  }
+  for (int i = 0; i < DPT; ++i) S[i] = (!fresh && col_on && d0 + i < D) ? st[(int64_t)(d0 + i) * p.V] : 0.0f;
   const float fixed = p.decay_kind == 1 ? p.decay[h] : 1.0f;
-  float nk[E], nq[E], na[E], nv[TB], nsc0 = 0.f, nsc1 = 1.f;
-  // request block b (tokens [b TB, b TB + TB)) into registers
-  auto request = [&](int b) {
+  float nk[E], nq[E], na[E], nv[TB], nsc0 = 0.f, nsc1 = fixed;
+  auto request = [&](int b) {  // block b (tokens [b TB, b TB + TB)) into registers
     const int t0 = b * TB;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
@@ -71,11 +79,12 @@ __global__ void matrix_scan_kernel(MatrixScanParams p, int R) {
       na[e] = (on && chan) ? p.decay[row * p.ldd + h * D + d] : 1.0f;
     }
 #pragma unroll
-    for (int t = 0; t < TB; ++t) nv[t] = (col_on && t0 + t < ql) ? p.v[(int64_t)(row0 + t0 + t) * p.ldv + h * p.V + j] : 0.0f;
+    for (int t = 0; t < TB; ++t)
+      nv[t] = (col_on && t0 + t < ql) ? p.v[(int64_t)(row0 + t0 + t) * p.ldv + h * p.V + j] : 0.0f;
     if (tid < TB && t0 + tid < ql) {
       const int64_t row = row0 + t0 + tid;
-      nsc0 = DELTA ? p.beta[row * p.ldb + h] : 0.0f;
-      nsc1 = p.decay_kind == 2 ? p.decay[row * p.ldd + h] : fixed;
+      if (DELTA) nsc0 = p.beta[row * p.ldb + h];
+      if (p.decay_kind == 2) nsc1 = p.decay[row * p.ldd + h];
     }
   };
   auto stage = [&](int buf) {
@@ -91,6 +100,43 @@ __global__ void matrix_scan_kernel(MatrixScanParams p, int R) {
       sc[(buf * 2 + 1) * TB + tid] = nsc1;
     }
   };
+  // one token: updates S, leaves this wave's share of the token's read-out in opart
+  auto token = [&](int buf, int t, float v) {
+    const float* kb = ks + (buf * TB + t) * Dp + d0;
+    const float* qb = qs + (buf * TB + t) * Dp + d0;
+    if (chan) {
+      const float* ab = as + (buf * TB + t) * Dp + d0;
+#pragma unroll
+      for (int i = 0; i < DPT; ++i) S[i] *= ab[i];
+    } else if (p.decay_kind != 0) {
+      const float sa = sc[(buf * 2 + 1) * TB + t];
+#pragma unroll
+      for (int i = 0; i < DPT; ++i) S[i] *= sa;
+    }
+    float u = v;
+    if (DELTA) {
+      float part = 0.f;
+#pragma unroll
+      for (int i = 0; i < DPT; ++i) part += S[i] * kb[i];
+      part = rows4_sum(part);  // the wave's RW rows
+      if (R > 1) {  // two alternating strips: a strip is rewritten two tokens later, after a barrier in between
+        float* ps = part_s + (t & 1) * R * kScanCols;
+        if (dg == 0) ps[r * kScanCols + c] = part;
+        lds_barrier();
+        part = 0.f;
+        for (int w = 0; w < R; ++w) part += ps[w * kScanCols + c];
+      }
+      u = sc[(buf * 2 + 0) * TB + t] * (v - part);
+    }
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < DPT; ++i) {
+      S[i] += kb[i] * u;
+      o += S[i] * qb[i];
+    }
+    o = rows4_sum(o);
+    if (dg == 0) opart[(t * R + r) * kScanCols + c] = o;
+  };
   const int nblocks = (ql + TB - 1) / TB;
   request(0);
   stage(0);
@@ -100,69 +146,41 @@ __global__ void matrix_scan_kernel(MatrixScanParams p, int R) {
 #pragma unroll
     for (int t = 0; t < TB; ++t) cv[t] = nv[t];
     if (b + 1 < nblocks) request(b + 1);  // in flight while this block is walked
-    __syncthreads();                      // this block's staging is visible; the previous block's opart has been read
+    lds_barrier();                        // this block's staging is visible; the previous block's opart has been read
     const int nt = ql - b * TB < TB ? ql - b * TB : TB;
+    if (nt == TB) {  // a full block: no branches between its tokens
 #pragma unroll
-    for (int t = 0; t < TB; ++t) {
-      if (t < nt) {  // uniform
-        const float* kb = ks + (buf * TB + t) * Dp + r * DPT;
-        const float* qb = qs + (buf * TB + t) * Dp + r * DPT;
-        if (chan) {
-          const float* ab = as + (buf * TB + t) * Dp + r * DPT;
+      for (int t = 0; t < TB; ++t) token(buf, t, cv[t]);
+    } else {
 #pragma unroll
-          for (int i = 0; i < DPT; ++i) S[i] *= ab[i];
-        } else if (p.decay_kind != 0) {
-          const float sa = sc[(buf * 2 + 1) * TB + t];
-#pragma unroll
-          for (int i = 0; i < DPT; ++i) S[i] *= sa;
-        }
-        float u = cv[t];
-        if (DELTA) {
-          float part = 0.f;
-#pragma unroll
-          for (int i = 0; i < DPT; ++i) part += S[i] * kb[i];
-          if (R > 1) {  // two alternating strips: a strip is rewritten two tokens later, after a barrier in between
-            float* ps = part_s + (t & 1) * R * kScanCols;
-            ps[r * kScanCols + lane] = part;
-            __syncthreads();
-            part = 0.f;
-            for (int w = 0; w < R; ++w) part += ps[w * kScanCols + lane];
-          }
-          u = sc[(buf * 2 + 0) * TB + t] * (cv[t] - part);
-        }
-        float o = 0.f;
-#pragma unroll
-        for (int i = 0; i < DPT; ++i) {
-          S[i] += kb[i] * u;
-          o += S[i] * qb[i];
-        }
-        opart[(t * R + r) * kScanCols + lane] = o;
-      }
+      for (int t = 0; t < TB; ++t)
+        if (t < nt) token(buf, t, cv[t]);  // uniform
     }
-    __syncthreads();  // the block's partial read-outs are complete; its staged inputs have been read
-    // token t of the block is finished by wave t mod R
-    for (int t = r; t < nt; t += R) {
+    lds_barrier();  // the block's partial read-outs are complete; its staged inputs have been read
+    // the block's [nt][16] outputs, one per thread
+    for (int idx = tid; idx < nt * kScanCols; idx += nthreads) {
+      const int t = idx / kScanCols, cc = idx % kScanCols;
       float o = 0.f;
-      for (int w = 0; w < R; ++w) o += opart[(t * R + w) * kScanCols + lane];
-      if (col_on) p.out[((int64_t)(row0 + b * TB + t) * p.H + h) * p.V + j] = o;
+      for (int w = 0; w < R; ++w) o += opart[(t * R + w) * kScanCols + cc];
+      const int jj = blockIdx.x * kScanCols + cc;
+      if (jj < p.V) p.out[((int64_t)(row0 + b * TB + t) * p.H + h) * p.V + jj] = o;
     }
     if (b + 1 < nblocks) stage(buf ^ 1);
   }
 #pragma unroll
-  for (int i = 0; i < DPT; ++i) {
-    const int d = r * DPT + i;
-    if (col_on && d < D) st[(int64_t)d * p.V] = S[i];
-  }
+  for (int i = 0; i < DPT; ++i)
+    if (col_on && d0 + i < D) st[(int64_t)(d0 + i) * p.V] = S[i];
 }
 
 template <int DPT, int TB>
 hipError_t launch(const MatrixScanParams& p, hipStream_t st) {
-  const int R = (p.D + DPT - 1) / DPT;
-  const int Dp = R * DPT;
+  constexpr int RW = 4 * DPT;
+  const int R = (p.D + RW - 1) / RW;
+  const int Dp = R * RW;
   dim3 grid((p.V + kScanCols - 1) / kScanCols, p.H, p.nseq);
   const size_t lds = (size_t)((p.decay_kind == 3 ? 6 : 4) * TB * Dp + 4 * TB + 2 * R * kScanCols + TB * R * kScanCols) *
                      sizeof(float);
-  if (lds > 64 * 1024) return hipErrorInvalidValue;
+  if (lds > 64 * 1024 || R > 16) return hipErrorInvalidValue;
   if (p.beta) hipLaunchKernelGGL((matrix_scan_kernel<DPT, TB, true>), grid, dim3(R * 64), lds, st, p, R);
   else hipLaunchKernelGGL((matrix_scan_kernel<DPT, TB, false>), grid, dim3(R * 64), lds, st, p, R);
   return hipGetLastError();
@@ -174,10 +192,10 @@ hipError_t launch(const MatrixScanParams& p, hipStream_t st) {
 extern "C" hipError_t dsse_matrix_scan(const dsse::MatrixScanParams* p, hipStream_t st) {
   if (p->nseq <= 0 || p->H <= 0) return hipSuccess;
   if (p->D < 1 || p->D > 512 || p->V < 1 || p->G < 1 || p->H % p->G) return hipErrorInvalidValue;
-  // rows of S per lane and tokens per block: more waves shorten the per-token chain (up to 16 waves per workgroup),
-  // the block is as long as 64 KB of LDS allow
-  if (p->D <= 64) return dsse::launch<8, 8>(*p, st);
-  if (p->D <= 128) return dsse::launch<16, 8>(*p, st);
-  if (p->D <= 256) return dsse::launch<16, 4>(*p, st);
-  return dsse::launch<32, 2>(*p, st);
+  // rows of S per lane (a wave holds 4 DPT rows of 16 columns, a workgroup up to 16 waves) and tokens per block (as
+  // long as 64 KB of LDS allow)
+  if (p->D <= 64) return dsse::launch<2, 16>(*p, st);
+  if (p->D <= 128) return dsse::launch<4, 16>(*p, st);
+  if (p->D <= 256) return dsse::launch<4, 8>(*p, st);
+  return dsse::launch<8, 4>(*p, st);
 }

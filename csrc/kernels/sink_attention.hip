@@ -146,13 +146,17 @@ __global__ __launch_bounds__(256) void sink_attention_kernel(SinkAttnParams p) {
 // lane group g are keys 4g..4g+3 of both 16-key halves, so the transposed page stores key k at position
 // 8 ((k & 15) >> 2) + 4 (k >> 4) + (k & 3).  The sink enters once, when the row is finished: it only enlarges the
 // denominator.
-template <int NT>  // V / 16 value tiles
+//
+// SPLIT (decode steps: few rows, long contexts): the four waves of a workgroup serve the SAME (tile, head) and take
+// every fourth page each; their (max, sum, O) are merged through LDS, so a sequence's keys are walked by four waves at
+// once and the launch has four times the waves.
+template <int NT, bool SPLIT>  // V / 16 value tiles
 __global__ __launch_bounds__(256) void sink_flash_kernel(SinkAttnParams p, const bf16* __restrict__ vt, int head_tiles) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   const int D = p.D, V = p.V;
   const int ldq = D + 8;  // bf16 elements per LDS row (16 B of padding)
   const int wave = threadIdx.x >> 6;
-  const int h = blockIdx.y * (blockDim.x >> 6) + wave;
+  const int h = SPLIT ? blockIdx.y : blockIdx.y * (blockDim.x >> 6) + wave;
   bf16* qs = reinterpret_cast<bf16*>(smem_raw) + wave * 16 * ldq;
   const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
   const int seq = p.work_seq[blockIdx.x], tile = p.work_tile[blockIdx.x];
@@ -178,7 +182,7 @@ __global__ __launch_bounds__(256) void sink_flash_kernel(SinkAttnParams p, const
     }
   }
   __syncthreads();
-  if (!h_ok) return;
+  if (!SPLIT && !h_ok) return;
   const int last_off = tile * 16 + 15 < ql ? tile * 16 + 15 : ql - 1;
   const int hi = pos0 + last_off;
   int lo = pos0 + tile * 16 - p.window + 1;
@@ -190,7 +194,7 @@ __global__ __launch_bounds__(256) void sink_flash_kernel(SinkAttnParams p, const
   for (int n = 0; n < NT; ++n) O[n] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
   const int nks = D / 32;
-  for (int pg = lo / kBS; pg <= hi / kBS; ++pg) {
+  for (int pg = lo / kBS + (SPLIT ? wave : 0); pg <= hi / kBS; pg += SPLIT ? 4 : 1) {
     int blk = bt[pg];
     blk = (unsigned)blk < (unsigned)p.num_blocks ? blk : 0;
     const bf16* krow0 = kc + (((int64_t)blk * kBS + r) * p.G + kvh) * D + 8 * g;  // key r of the page's first half
@@ -247,6 +251,39 @@ __global__ __launch_bounds__(256) void sink_flash_kernel(SinkAttnParams p, const
       O[n] = mfma16x16x32(vf[n], pf, o);
     }
   }
+  if (SPLIT) {
+    // merge the four waves' partial results: [wave][16 columns][V + 2] floats, after every wave has read its queries
+    float* mg = reinterpret_cast<float*>(smem_raw) + 4 * 16 * ((ldq + 1) / 2);
+    const int ldm = V + 2;
+    float* mine = mg + (wave * 16 + r) * ldm;
+#pragma unroll
+    for (int n = 0; n < NT; ++n)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mine[16 * n + 4 * g + i] = O[n][i];
+    if (g == 0) {
+      mine[V] = m;
+      mine[V + 1] = l;
+    }
+    __syncthreads();
+    const int rows_on = ql - tile * 16 < 16 ? ql - tile * 16 : 16;
+    for (int idx = threadIdx.x; idx < rows_on * V; idx += blockDim.x) {
+      const int col = idx / V, d = idx - col * V;
+      const int64_t row = q0 + tile * 16 + col;
+      float mm = p.sink ? p.sink[h] : -INFINITY;
+      for (int w = 0; w < 4; ++w) mm = fmaxf(mm, mg[(w * 16 + col) * ldm + V]);
+      float den = p.sink ? expf(p.sink[h] - mm) : 0.f, num = 0.f;
+      for (int w = 0; w < 4; ++w) {
+        const float* src = mg + (w * 16 + col) * ldm;
+        const float f = src[V] == -INFINITY ? 0.f : expf(src[V] - mm);
+        den += src[V + 1] * f;
+        num += src[d] * f;
+      }
+      float o = den > 0.f ? num / den : 0.f;
+      if (p.gate) o *= 1.0f / (1.0f + expf(-p.gate[row * p.ldg + h]));
+      reinterpret_cast<bf16*>(p.out)[(row * p.H + h) * V + d] = (bf16)o;
+    }
+    return;
+  }
   if (c_ok) {
     float den = l, f = 1.0f;
     if (p.sink) {  // the sink joins the denominator under the common maximum
@@ -269,23 +306,30 @@ __global__ __launch_bounds__(256) void sink_flash_kernel(SinkAttnParams p, const
 }
 
 template <int NT>
-void launch_flash(int num_work, const SinkAttnParams& p, const bf16* vt, hipStream_t st) {
+void launch_flash(int num_work, const SinkAttnParams& p, const bf16* vt, int split, hipStream_t st) {
+  const size_t qbytes = 16 * (size_t)(p.D + 8) * sizeof(bf16);
+  if (split) {  // one head per workgroup, its four waves share the keys; LDS: 4 query tiles + the merge area
+    const size_t lds = 4 * 16 * (size_t)((p.D + 8 + 1) / 2) * sizeof(float) + 4 * 16 * (size_t)(p.V + 2) * sizeof(float);
+    hipLaunchKernelGGL((sink_flash_kernel<NT, true>), dim3(num_work, p.H), dim3(256), lds, st, p, vt, p.H);
+    return;
+  }
   const int wy = p.H < 4 ? p.H : 4;
-  const size_t lds = wy * 16 * (size_t)(p.D + 8) * sizeof(bf16);
   dim3 grid(num_work, (p.H + wy - 1) / wy), block(64 * wy);
-  hipLaunchKernelGGL(sink_flash_kernel<NT>, grid, block, lds, st, p, vt, p.H);
+  hipLaunchKernelGGL((sink_flash_kernel<NT, false>), grid, block, wy * qbytes, st, p, vt, p.H);
 }
 
 }  // namespace
 }  // namespace dsse
 
 // work_tile counts tiles of 16 rows; vt: transposed value pages [pages, G, V, kBS], keys permuted inside a page
-extern "C" hipError_t dsse_sink_flash(int num_work, const dsse::SinkAttnParams* p, const void* vt, hipStream_t st) {
+extern "C" hipError_t dsse_sink_flash(int num_work, const dsse::SinkAttnParams* p, const void* vt, int split,
+                                      hipStream_t st) {
   if (num_work <= 0 || p->H <= 0) return hipSuccess;
   if (p->f32 || p->D % 32 || p->V % 16 || p->V > 512 || p->D > 512 || p->H % p->G) return hipErrorInvalidValue;
+  if (split && p->V > 128) return hipErrorInvalidValue;  // the merge area has to fit 64 KB of LDS
   const bf16* v = reinterpret_cast<const bf16*>(vt);
   switch (p->V / 16) {
-#define DSSE_FLASH_CASE(n) case n: dsse::launch_flash<n>(num_work, *p, v, st); break;
+#define DSSE_FLASH_CASE(n) case n: dsse::launch_flash<n>(num_work, *p, v, split, st); break;
     DSSE_FLASH_CASE(1) DSSE_FLASH_CASE(2) DSSE_FLASH_CASE(3) DSSE_FLASH_CASE(4) DSSE_FLASH_CASE(5) DSSE_FLASH_CASE(6)
     DSSE_FLASH_CASE(7) DSSE_FLASH_CASE(8) DSSE_FLASH_CASE(10) DSSE_FLASH_CASE(12) DSSE_FLASH_CASE(16)
     DSSE_FLASH_CASE(20) DSSE_FLASH_CASE(24) DSSE_FLASH_CASE(32)

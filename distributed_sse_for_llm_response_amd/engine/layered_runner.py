@@ -392,6 +392,9 @@ class LayeredRunner(RunnerBase):
             if vt is not None and g["qt"] > 1:  # prompt portions on the MFMA form: tiles of 16 rows
                 ops.sink_attention(qa, self.kv.k[ri], self.kv.v[ri], g["bt"], g["qs"], g["ql"], g["ctx"], g["hs"],
                                    g["ht"], Lw.sink, small[:, :H], ao, a.window, a.scale, SINK_ROWS_TILE, vt)
+            elif vt is not None and V <= ops.layers.SINK_SPLIT_MAX_V:  # decode rows: tile 0, keys split over the waves
+                ops.sink_attention(qa, self.kv.k[ri], self.kv.v[ri], g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"],
+                                   g["wt"], Lw.sink, small[:, :H], ao, a.window, a.scale, SINK_ROWS_TILE, vt, True)
             else:
                 ops.sink_attention(qa, self.kv.k[ri], self.kv.v[ri], g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"],
                                    g["wt"], Lw.sink, small[:, :H], ao, a.window, a.scale, g["qt"])

@@ -172,20 +172,24 @@ def norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind: int, ep
 SINK_FLASH_TILES = (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16, 20, 24, 32)  # value widths / 16 the MFMA form is built for
 
 
+SINK_SPLIT_MAX_V = 128  # widest value head whose key-split merge area fits LDS
+
+
 def sink_flash_ok(dtype, dim: int, vdim: int) -> bool:
     """Shapes the MFMA form of sink_attention covers (prompt portions; everything else takes the row kernel)."""
     return dtype == torch.bfloat16 and dim % 32 == 0 and dim <= 512 and vdim % 16 == 0 and vdim // 16 in SINK_FLASH_TILES
 
 
 def sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile, sink, gate, out,
-                   window: int, scale: float, qt: int, vt=None):
+                   window: int, scale: float, qt: int, vt=None, split: bool = False):
     """Causal softmax attention of q [T, H, D] over paged keys [pages, 32, G, D] and values [pages, 32, G, V] (grouped
     heads), scores and weights in fp32; sink [H] adds exp(sink) to each head's denominator, gate [T, H] multiplies the
     head's output by its sigmoid.  `qt` query rows per work item (work_seq, work_tile).  With vt (transposed value
-    pages [pages, G, V, 32], sink_flash_ok shapes, qt = 16): the MFMA form for prompt portions."""
+    pages [pages, G, V, 32], sink_flash_ok shapes, qt = 16): the MFMA form; split (V <= 128) lets the four waves of a
+    workgroup share one (tile, head) and split its pages, for decode steps."""
     if _hip(q):
         torch.ops.dsse.sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile,
-                                      sink, gate, out, window, scale, qt, vt)
+                                      sink, gate, out, window, scale, qt, vt, split)
     else:
         lref.sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, sink, gate, out, window, scale, vt)
 
