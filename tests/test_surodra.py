@@ -483,3 +483,16 @@ def test_config_round_trip_and_registry(tmp_path):
     bad["l0.mix.q"] = bad["l0.mix.q"][:-1]
     with pytest.raises(ValueError):
         convert_surodra(cfg, bad)
+
+
+def test_serving_builds_the_family_by_name():
+    """The serving launcher's engine builder resolves the family through the registry and generates with it."""
+    from distributed_sse_for_llm_response_amd.serving.app import build_engine
+    from distributed_sse_for_llm_response_amd.serving.config import ServeConfig
+
+    eng, _ = build_engine(ServeConfig(model="surodra-tiny", engine="cpu"))
+    eng.add_request("c1", [5, 6, 7, 8, 9, 10], SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))
+    eng.add_request("c2", [11, 12], SamplingParams(temperature=0.8, max_tokens=3, ignore_eos=True))
+    ev = eng.run_until_idle()
+    assert sum(1 for e in ev if e.conversation_id == "c1" and not e.done) == 4
+    assert sum(1 for e in ev if e.conversation_id == "c2" and not e.done) == 3
