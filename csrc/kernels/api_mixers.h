@@ -76,6 +76,30 @@ struct MatrixScanParams {
   int nseq, H, G, D, V, ldq, ldk, ldv, ldd, ldb;
   int decay_kind;        // 0 none
   float q_scale;
+  // two-level walk of long prompt portions (src_idx null = the plain walk): a "sequence" of the launch is then a CHUNK
+  // of a portion, its initial state comes from entry src_idx[i] of `src` (-1 = zeros) and its end state goes to entry
+  // dst_idx[i] of `dst` (-1 = nowhere); entries are [H, D, V]
+  const int* src_idx;
+  const int* dst_idx;
+  const float* src;
+  float* dst;
+  int no_out;            // 1: a pass that only produces end states
+  float* a_out;          // [nseq, H, D] product of the chunk's per-channel decays (decay_kind 3) or null
+};
+
+// The carry between the two passes of the two-level walk: per sequence, the incoming state of each of its chunks.
+struct ScanCarryParams {
+  float* scratch;        // [chunks, H, D, V]: in: a chunk's end state from zeros; out: the chunk's incoming state
+  const float* a_chunk;  // [chunks, H, D] per-channel decay products (decay_kind 3) or null
+  const float* decay;    // [H] (decay_kind 1) or null
+  const float* state;    // [slots, H, D, V]
+  const int* q_len;      // per sequence
+  const int* ctx_len;
+  const int* state_slot;
+  const int* s_first;    // first chunk of the sequence
+  const int* s_count;    // its chunks
+  const int* cq_len;     // [chunks] tokens of a chunk
+  int nseq, H, D, V, decay_kind;
 };
 
 }  // namespace dsse
@@ -92,6 +116,7 @@ hipError_t dsse_sink_flash(int num_work, const dsse::SinkAttnParams* p, const vo
 hipError_t dsse_gate_math(float* x, int ld, int M, int N, int kind, const float* p1, const float* p2, float c,
                           hipStream_t st);
 hipError_t dsse_matrix_scan(const dsse::MatrixScanParams* p, hipStream_t st);
+hipError_t dsse_scan_carry(const dsse::ScanCarryParams* p, hipStream_t st);
 hipError_t dsse_gated_head_norm(const float* o, const float* w, const float* gate, int ldg, void* out, int M, int H,
                                 int V, float eps, int f32, hipStream_t st);
 hipError_t dsse_rms_mix(const float* ya, const float* wa, const float* yb, const float* wb, float* out, int M, int W,

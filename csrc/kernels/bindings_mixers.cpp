@@ -304,6 +304,95 @@ void matrix_scan(const Tensor& q, const Tensor& k, const Tensor& v, const OptTen
   DSSE_CHECK_HIP(dsse_matrix_scan(&p, cur_stream()));
 }
 
+// Two-level walk of long prompt portions without the delta rule: (1) every chunk but a sequence's last is walked from
+// zeros and leaves its end state in `scratch`; (2) the carry turns those into each chunk's incoming state; (3) every
+// chunk is walked from its incoming state and writes its outputs, the last chunk of a sequence also the slot's state.
+// cmeta [7, chunks]: first row, tokens, tokens in pass 1 (0 for a sequence's last chunk), -1s, pass-1 destination
+// (own entry or -1), own entry, pass-3 destination (the state slot for a sequence's last chunk, else -1).
+void matrix_scan_chunked(const Tensor& q, const Tensor& k, const Tensor& v, const OptTensor& decay, Tensor& state,
+                         const Tensor& q_len, const Tensor& ctx_len, const Tensor& state_slot, const Tensor& s_first,
+                         const Tensor& s_count, const Tensor& cmeta, Tensor& scratch, const OptTensor& a_scratch,
+                         Tensor& out, double q_scale) {
+  head_view(q, "q");
+  head_view(k, "k");
+  head_view(v, "v");
+  f32t(state, "state");
+  f32t(out, "out");
+  f32t(scratch, "scratch");
+  i32(cmeta, "cmeta");
+  i32(q_len, "q_len");
+  i32(ctx_len, "ctx_len");
+  i32(state_slot, "state_slot");
+  i32(s_first, "s_first");
+  i32(s_count, "s_count");
+  dsse::MatrixScanParams p{};
+  const int T = (int)v.size(0);
+  p.H = (int)v.size(1), p.V = (int)v.size(2), p.G = (int)k.size(1), p.D = (int)k.size(2);
+  TORCH_CHECK(q.sizes() == k.sizes() && q.size(0) == T && p.G >= 1 && p.H % p.G == 0 && p.D <= 512, "q, k [T, G, D], v [T, H, V]");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == p.H && state.size(2) == p.D && state.size(3) == p.V,
+              "state must be [slots, H, D, V]");
+  TORCH_CHECK(out.dim() == 3 && out.sizes() == v.sizes(), "out must be [T, H, V]");
+  TORCH_CHECK(cmeta.dim() == 2 && cmeta.size(0) == 7, "cmeta must be [7, chunks]");
+  const int N = (int)cmeta.size(1), ns = (int)q_len.numel();
+  const int64_t entry = (int64_t)p.H * p.D * p.V;
+  TORCH_CHECK(scratch.numel() >= N * entry, "scratch must hold [chunks, H, D, V]");
+  TORCH_CHECK(ctx_len.numel() >= ns && state_slot.numel() >= ns && s_first.numel() >= ns && s_count.numel() >= ns &&
+                  N <= 65535 && ns <= 65535,
+              "sequence metadata too short / too many chunks");
+  p.q = q.data_ptr<float>(), p.k = k.data_ptr<float>(), p.v = v.data_ptr<float>();
+  p.ldq = (int)q.stride(0), p.ldk = (int)k.stride(0), p.ldv = (int)v.stride(0);
+  dsse::ScanCarryParams cp{};
+  if (decay.has_value()) {
+    const Tensor& d = *decay;
+    f32t(d, "decay", false);
+    if (d.dim() == 1) {
+      TORCH_CHECK(d.size(0) == p.H && (p.H == 1 || d.stride(0) == 1), "decay [H]");
+      p.decay_kind = 1;
+      cp.decay = d.data_ptr<float>();
+    } else {
+      head_view(d, "decay");
+      TORCH_CHECK(d.dim() == 3 && d.size(0) == T && d.size(1) == p.H && d.size(2) == p.D, "decay [T, H, D]");
+      TORCH_CHECK(a_scratch.has_value(), "per-channel decays need a_scratch");
+      f32t(*a_scratch, "a_scratch");
+      TORCH_CHECK(a_scratch->numel() >= (int64_t)N * p.H * p.D, "a_scratch must hold [chunks, H, D]");
+      p.decay_kind = 3;
+      p.ldd = (int)d.stride(0);
+      p.a_out = a_scratch->data_ptr<float>();
+      cp.a_chunk = p.a_out;
+    }
+    p.decay = d.data_ptr<float>();
+  }
+  const int* cm = cmeta.data_ptr<int>();
+  p.state = state.data_ptr<float>();
+  p.nseq = N;
+  p.q_start = cm;
+  p.ctx_len = cm + N;  // unused by the chunked walk (src_idx decides where a chunk starts from)
+  p.state_slot = cm + 5 * N;
+  p.out = out.data_ptr<float>();
+  p.q_scale = (float)q_scale;
+  // pass 1: from zeros, end states into scratch
+  p.q_len = cm + 2 * N;
+  p.src_idx = cm + 3 * N, p.dst_idx = cm + 4 * N;
+  p.src = scratch.data_ptr<float>(), p.dst = scratch.data_ptr<float>();
+  p.no_out = 1;
+  DSSE_CHECK_HIP(dsse_matrix_scan(&p, cur_stream()));
+  // carry
+  cp.scratch = scratch.data_ptr<float>();
+  cp.state = state.data_ptr<float>();
+  cp.q_len = q_len.data_ptr<int>(), cp.ctx_len = ctx_len.data_ptr<int>(), cp.state_slot = state_slot.data_ptr<int>();
+  cp.s_first = s_first.data_ptr<int>(), cp.s_count = s_count.data_ptr<int>();
+  cp.cq_len = cm + N;
+  cp.nseq = ns, cp.H = p.H, cp.D = p.D, cp.V = p.V, cp.decay_kind = p.decay_kind;
+  DSSE_CHECK_HIP(dsse_scan_carry(&cp, cur_stream()));
+  // pass 2: from the incoming states, outputs; a sequence's last chunk leaves the slot's state
+  p.q_len = cm + N;
+  p.src_idx = cm + 5 * N, p.dst_idx = cm + 6 * N;
+  p.dst = state.data_ptr<float>();
+  p.no_out = 0;
+  p.a_out = nullptr;
+  DSSE_CHECK_HIP(dsse_matrix_scan(&p, cur_stream()));
+}
+
 void gated_head_norm(const Tensor& o, const OptTensor& w, const Tensor& gate, double eps, Tensor& out) {
   f32t(o, "o");
   col_view(gate, "gate");
@@ -350,6 +439,9 @@ TORCH_LIBRARY_FRAGMENT(dsse, m) {
   m.def("gate_math(Tensor(a!) x, int kind, Tensor? p1=None, Tensor? p2=None, float c=1.0) -> ()");
   m.def("matrix_scan(Tensor q, Tensor k, Tensor v, Tensor? decay, Tensor? beta, Tensor(a!) state, Tensor q_start, "
         "Tensor q_len, Tensor ctx_len, Tensor state_slot, Tensor(b!) out, float q_scale=1.0) -> ()");
+  m.def("matrix_scan_chunked(Tensor q, Tensor k, Tensor v, Tensor? decay, Tensor(a!) state, Tensor q_len, Tensor ctx_len, "
+        "Tensor state_slot, Tensor s_first, Tensor s_count, Tensor cmeta, Tensor(b!) scratch, Tensor(c!)? a_scratch, "
+        "Tensor(d!) out, float q_scale=1.0) -> ()");
   m.def("gated_head_norm(Tensor o, Tensor? w, Tensor gate, float eps, Tensor(a!) out) -> ()");
   m.def("rms_mix(Tensor ya, Tensor wa, Tensor yb, Tensor wb, float eps, float coef, Tensor(a!) out) -> ()");
   m.def("logit_cap(Tensor(a!) logits, float scale, float cap) -> ()");
@@ -362,6 +454,7 @@ TORCH_LIBRARY_IMPL(dsse, CUDA, m) {
   m.impl("sink_attention", &sink_attention);
   m.impl("gate_math", &gate_math);
   m.impl("matrix_scan", &matrix_scan);
+  m.impl("matrix_scan_chunked", &matrix_scan_chunked);
   m.impl("gated_head_norm", &gated_head_norm);
   m.impl("rms_mix", &rms_mix);
   m.impl("logit_cap", &logit_cap);

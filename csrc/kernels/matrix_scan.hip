@@ -59,11 +59,24 @@ __global__ __launch_bounds__(1024) void matrix_scan_kernel(MatrixScanParams p, i
   float* part_s = sc + 4 * TB;
   float* opart = part_s + 2 * R * kScanCols;
   const int row0 = p.q_start[seq];
-  const bool fresh = p.ctx_len[seq] - ql == 0;
-  float* st = p.state + (((int64_t)p.state_slot[seq] * p.H + h) * D) * p.V + j;
-  float S[DPT];
+  // where the walk starts from and where its end state goes: the sequence's slot (zeros at position 0), or, for a
+  // chunk of the two-level walk, the entries its lists name
+  const float* from;
+  float* to;
+  if (p.src_idx) {
+    const int si = p.src_idx[seq], di = p.dst_idx[seq];
+    from = si >= 0 ? p.src + (((int64_t)si * p.H + h) * D) * p.V + j : nullptr;
+    to = di >= 0 ? p.dst + (((int64_t)di * p.H + h) * D) * p.V + j : nullptr;
+  } else {
+    to = p.state + (((int64_t)p.state_slot[seq] * p.H + h) * D) * p.V + j;
+    from = p.ctx_len[seq] - ql == 0 ? nullptr : to;
+  }
+  float S[DPT], P[DPT];
 #pragma unroll
-  for (int i = 0; i < DPT; ++i) S[i] = (!fresh && col_on && d0 + i < D) ? st[(int64_t)(d0 + i) * p.V] : 0.0f;
+  for (int i = 0; i < DPT; ++i) {
+    S[i] = (from && col_on && d0 + i < D) ? from[(int64_t)(d0 + i) * p.V] : 0.0f;
+    P[i] = 1.0f;
+  }
   const float fixed = p.decay_kind == 1 ? p.decay[h] : 1.0f;
   float nk[E], nq[E], na[E], nv[TB], nsc0 = 0.f, nsc1 = fixed;
   auto request = [&](int b) {  // block b (tokens [b TB, b TB + TB)) into registers
@@ -108,6 +121,10 @@ __global__ __launch_bounds__(1024) void matrix_scan_kernel(MatrixScanParams p, i
       const float* ab = as + (buf * TB + t) * Dp + d0;
 #pragma unroll
       for (int i = 0; i < DPT; ++i) S[i] *= ab[i];
+      if (p.a_out) {  // uniform: the chunk's decay product for the carry
+#pragma unroll
+        for (int i = 0; i < DPT; ++i) P[i] *= ab[i];
+      }
     } else if (p.decay_kind != 0) {
       const float sa = sc[(buf * 2 + 1) * TB + t];
 #pragma unroll
@@ -158,7 +175,7 @@ __global__ __launch_bounds__(1024) void matrix_scan_kernel(MatrixScanParams p, i
     }
     lds_barrier();  // the block's partial read-outs are complete; its staged inputs have been read
     // the block's [nt][16] outputs, one per thread
-    for (int idx = tid; idx < nt * kScanCols; idx += nthreads) {
+    for (int idx = tid; idx < (p.no_out ? 0 : nt * kScanCols); idx += nthreads) {
       const int t = idx / kScanCols, cc = idx % kScanCols;
       float o = 0.f;
       for (int w = 0; w < R; ++w) o += opart[(t * R + w) * kScanCols + cc];
@@ -167,9 +184,45 @@ __global__ __launch_bounds__(1024) void matrix_scan_kernel(MatrixScanParams p, i
     }
     if (b + 1 < nblocks) stage(buf ^ 1);
   }
+  if (to) {
 #pragma unroll
-  for (int i = 0; i < DPT; ++i)
-    if (col_on && d0 + i < D) st[(int64_t)(d0 + i) * p.V] = S[i];
+    for (int i = 0; i < DPT; ++i)
+      if (col_on && d0 + i < D) to[(int64_t)(d0 + i) * p.V] = S[i];
+  }
+  if (p.a_out && chan && blockIdx.x == 0 && c == 0) {
+#pragma unroll
+    for (int i = 0; i < DPT; ++i)
+      if (d0 + i < D) p.a_out[((int64_t)seq * p.H + h) * D + d0 + i] = P[i];
+  }
+}
+
+// S_in of every chunk of a sequence: S_in[0] = the slot's state (zeros at position 0), S_in[c + 1] = A_c S_in[c] + B_c
+// with B_c the chunk's end state from zeros (found in its scratch entry, which then receives S_in[c]) and A_c the
+// product of its decays.  One thread per state element; a sequence has a handful of chunks.
+__global__ __launch_bounds__(256) void scan_carry_kernel(ScanCarryParams p) {
+  const int seq = blockIdx.z, h = blockIdx.y;
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t DV = (int64_t)p.D * p.V;
+  const int n = p.s_count[seq];
+  if (e >= DV || n <= 0 || p.q_len[seq] <= 0) return;
+  const int d = (int)(e / p.V);
+  const bool fresh = p.ctx_len[seq] - p.q_len[seq] == 0;
+  float S = fresh ? 0.0f : p.state[((int64_t)p.state_slot[seq] * p.H + h) * DV + e];
+  const float fixed = p.decay_kind == 1 ? p.decay[h] : 1.0f;
+  const int c0 = p.s_first[seq];
+  for (int i = 0; i < n; ++i) {
+    const int cid = c0 + i;
+    float* slot = p.scratch + ((int64_t)cid * p.H + h) * DV + e;
+    const float B = *slot;
+    *slot = S;
+    if (i + 1 < n) {
+      float a = 1.0f;
+      if (p.decay_kind == 3) a = p.a_chunk[((int64_t)cid * p.H + h) * p.D + d];
+      else if (p.decay_kind == 1)
+        for (int t = 0; t < p.cq_len[cid]; ++t) a *= fixed;  // the product the walk itself would form
+      S = a * S + B;
+    }
+  }
 }
 
 template <int DPT, int TB>
@@ -198,4 +251,11 @@ extern "C" hipError_t dsse_matrix_scan(const dsse::MatrixScanParams* p, hipStrea
   if (p->D <= 128) return dsse::launch<4, 16>(*p, st);
   if (p->D <= 256) return dsse::launch<4, 8>(*p, st);
   return dsse::launch<8, 4>(*p, st);
+}
+
+extern "C" hipError_t dsse_scan_carry(const dsse::ScanCarryParams* p, hipStream_t st) {
+  if (p->nseq <= 0 || p->H <= 0) return hipSuccess;
+  const long long dv = (long long)p->D * p->V;
+  hipLaunchKernelGGL(dsse::scan_carry_kernel, dim3((unsigned)((dv + 255) / 256), p->H, p->nseq), dim3(256), 0, st, *p);
+  return hipGetLastError();
 }

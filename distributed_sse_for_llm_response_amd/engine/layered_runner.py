@@ -336,6 +336,13 @@ class LayeredRunner(RunnerBase):
         ops.gated_act(gu, h, 1)
         self._lin(h, Fw.down, Fw.down_t, d["y"])
 
+    def _scratch(self, d: dict, name: str, numel: int):
+        """An fp32 work area of the step, grown on demand and shared by its layers."""
+        t = d.get(name)
+        if t is None or t.numel() < numel:
+            t = d[name] = torch.empty(numel, device=self.device, dtype=torch.float32)
+        return t
+
     @staticmethod
     def _cols(buf, c0: int, heads: int, width: int):
         """Columns [c0, c0 + heads * width) of a row-major fp32 buffer as [rows, heads, width] (a view)."""
@@ -346,7 +353,16 @@ class LayeredRunner(RunnerBase):
         """Recurrence over every sequence group, per-head output norm times the SiLU gate, output projection."""
         o = d["o"][:M * H * V].view(M, H, V)
         for g in groups:
-            ops.matrix_scan(q, k, v, decay, beta, self.state.state[ri], g["qs"], g["ql"], g["ctx"], g["ss"], o, q_scale)
+            if beta is None and "ck" in g:
+                s_first, s_count, cm = g["ck"]
+                D = k.shape[2]
+                scr = self._scratch(d, "scan_s", cm.shape[1] * H * D * V)
+                ascr = self._scratch(d, "scan_a", cm.shape[1] * H * D) if decay is not None and decay.dim() == 3 else None
+                ops.matrix_scan_chunked(q, k, v, decay, self.state.state[ri], g["qs"], g["ql"], g["ctx"], g["ss"],
+                                        s_first, s_count, cm, scr, ascr, o, q_scale)
+            else:
+                ops.matrix_scan(q, k, v, decay, beta, self.state.state[ri], g["qs"], g["ql"], g["ctx"], g["ss"], o,
+                                q_scale)
         ao = d["ao"][:M * H * V].view(M, H * V)
         ops.gated_head_norm(o, Lw_norm, gate, self.cfg.eps, ao)
         self._lin(ao, o_w, o_t, y)
@@ -521,6 +537,14 @@ class LayeredRunner(RunnerBase):
             d[name], o = meta[o:o + k], o + k
         d["bt"] = bt
         d["qt"] = ATTN_ROWS_TILE
+        if self.prenorm and T >= ops.layers.SCAN_CHUNKED_FROM:  # long portions: the recurrences' two-level walk
+            s_first, s_count, rows = ops.layers.scan_chunks(qs, ql, ss)
+            ck = torch.tensor([s_first, s_count], dtype=torch.int32)
+            cm = torch.tensor(rows, dtype=torch.int32)
+            if self.device.type == "cuda":
+                ck = ck.pin_memory().to(self.device, non_blocking=True)
+                cm = cm.pin_memory().to(self.device, non_blocking=True)
+            d["ck"] = (ck[0], ck[1], cm)
         return T, qs, ql, d
 
     def prefill(self, seqs: list, ring_row: int, trace: list | None = None) -> None:

@@ -213,6 +213,41 @@ def matrix_scan(q, k, v, decay, beta, state, q_start, q_len, ctx_len, state_slot
         lref.matrix_scan(q, k, v, decay, beta, state, q_start, q_len, ctx_len, state_slot, out, q_scale)
 
 
+SCAN_CHUNK = 64        # tokens per chunk of the two-level walk
+SCAN_CHUNKED_FROM = 256  # rows of a prompt group from which matrix_scan_chunked pays
+
+
+def scan_chunks(q_start: list, q_len: list, slots: list):
+    """Host-side chunk lists of matrix_scan_chunked for sequences with the given first rows, lengths and state slots:
+    (s_first, s_count, cmeta [7][chunks]) as Python lists (see the op for cmeta's rows)."""
+    s_first, s_count = [], []
+    rows = [[] for _ in range(7)]
+    for r0, n, slot in zip(q_start, q_len, slots):
+        k = -(-n // SCAN_CHUNK) if n > 0 else 0
+        s_first.append(len(rows[0]))
+        s_count.append(k)
+        for i in range(k):
+            cid, last = len(rows[0]), i == k - 1
+            ln = min(SCAN_CHUNK, n - i * SCAN_CHUNK)
+            for row, val in zip(rows, (r0 + i * SCAN_CHUNK, ln, 0 if last else ln, -1, -1 if last else cid, cid,
+                                       slot if last else -1)):
+                row.append(val)
+    return s_first, s_count, rows
+
+
+def matrix_scan_chunked(q, k, v, decay, state, q_start, q_len, ctx_len, state_slot, s_first, s_count, cmeta, scratch,
+                        a_scratch, out, q_scale: float = 1.0):
+    """matrix_scan without the delta rule for long prompt portions, as a two-level walk: chunks of SCAN_CHUNK tokens are
+    walked in parallel from zeros, a carry gives every chunk its incoming state, and a second parallel walk writes the
+    outputs and the slots' states.  decay: None, [H] or [T, H, D].  Chunk lists from scan_chunks; scratch
+    [chunks, H, D, V] and a_scratch [chunks, H, D] (per-channel decays) are fp32 work areas."""
+    if _hip(v):
+        torch.ops.dsse.matrix_scan_chunked(q, k, v, decay, state, q_len, ctx_len, state_slot, s_first, s_count, cmeta,
+                                           scratch, a_scratch, out, q_scale)
+    else:
+        lref.matrix_scan(q, k, v, decay, None, state, q_start, q_len, ctx_len, state_slot, out, q_scale)
+
+
 def gated_head_norm(o, w, gate, eps: float, out):
     """out [T, H * V] (element type) = o / rms(o) per head * w (or no gain) * silu(gate)."""
     if _hip(o):

@@ -282,3 +282,36 @@ def test_conv_state_strided_silu():
     ops.conv_state(c(wide)[:, 3:3 + C], c(taps), None, tl, c(qs), c(i32(ql)), c(i32(ctx)), c(i32(slot)), o, None, None, 1)
     close(o, o_ref, 2e-6)
     close(tl, t_ref, 1e-6)
+
+
+@pytest.mark.parametrize("H,G,D,V", [(3, 1, 32, 40), (2, 2, 128, 64), (1, 1, 72, 16)])
+@pytest.mark.parametrize("mode", ["channel", "fixed", "plain"])
+def test_matrix_scan_two_level_walk(H, G, D, V, mode):
+    """Long portions walked in chunks (parallel from zeros, carry, parallel again) against the plain reference walk:
+    a fresh prompt that ends inside a chunk, a later portion continued from its slot, one exactly one chunk long, one
+    shorter than a chunk."""
+    from distributed_sse_for_llm_response_amd.ops.layers import scan_chunks
+
+    g = torch.Generator().manual_seed(11)
+    ql, ctx, slot = [200, 131, 64, 5], [200, 300, 64, 90], [2, 0, 3, 1]
+    qs = [0, 200, 331, 395]
+    T = sum(ql)
+    q = torch.randn(T, G, D, generator=g) * 0.3
+    k = torch.randn(T, G, D, generator=g) * 0.3
+    v = torch.randn(T, H, V, generator=g)
+    decay = {"channel": torch.rand(T, H, D, generator=g) * 0.1 + 0.9, "fixed": torch.linspace(0.9, 0.999, H),
+             "plain": None}[mode]
+    state0 = torch.randn(4, H, D, V, generator=g)
+    st_ref, o_ref = state0.clone(), torch.zeros(T, H, V)
+    lref.matrix_scan(q, k, v, decay, None, st_ref, i32(qs), i32(ql), i32(ctx), i32(slot), o_ref, 0.5)
+    s_first, s_count, rows = scan_chunks(qs, ql, slot)
+    assert s_count == [4, 3, 1, 1]
+    c = lambda t: None if t is None else t.to(dev())  # noqa: E731
+    st, o = c(state0.clone()), torch.zeros(T, H, V, device=dev())
+    n = len(rows[0])
+    scr = torch.full((n * H * D * V,), float("nan"), device=dev())
+    ascr = torch.full((n * H * D,), float("nan"), device=dev()) if mode == "channel" else None
+    ops.matrix_scan_chunked(c(q), c(k), c(v), c(decay), st, c(i32(qs)), c(i32(ql)), c(i32(ctx)), c(i32(slot)),
+                            c(i32(s_first)), c(i32(s_count)), c(i32(rows)), scr, ascr, o, 0.5)
+    close(o, o_ref, 3e-5)
+    close(st, st_ref, 3e-5)
