@@ -61,20 +61,27 @@ __global__ __launch_bounds__(1024) void matrix_scan_kernel(MatrixScanParams p, i
   const int row0 = p.q_start[seq];
   // where the walk starts from and where its end state goes: the sequence's slot (zeros at position 0), or, for a
   // chunk of the two-level walk, the entries its lists name
+  // State entries [H, D, V] are kept tile-major when V is a multiple of 16 -- [H][V / 16][D][16], a workgroup's 16
+  // columns contiguous -- so that every 128-byte line of the state is read and written by ONE workgroup; in the
+  // plain layout two workgroups (often on different L2s) would each pull the whole line for their 64 bytes of it.
+  const bool tiled = p.V % kScanCols == 0;
+  const int64_t rs = tiled ? kScanCols : p.V;  // floats between two rows of this lane's column
+  const int64_t col_off = tiled ? (int64_t)blockIdx.x * D * kScanCols + c : j;
+  const int64_t entry = (int64_t)p.H * D * p.V;
   const float* from;
   float* to;
   if (p.src_idx) {
     const int si = p.src_idx[seq], di = p.dst_idx[seq];
-    from = si >= 0 ? p.src + (((int64_t)si * p.H + h) * D) * p.V + j : nullptr;
-    to = di >= 0 ? p.dst + (((int64_t)di * p.H + h) * D) * p.V + j : nullptr;
+    from = si >= 0 ? p.src + si * entry + (int64_t)h * D * p.V + col_off : nullptr;
+    to = di >= 0 ? p.dst + di * entry + (int64_t)h * D * p.V + col_off : nullptr;
   } else {
-    to = p.state + (((int64_t)p.state_slot[seq] * p.H + h) * D) * p.V + j;
+    to = p.state + p.state_slot[seq] * entry + (int64_t)h * D * p.V + col_off;
     from = p.ctx_len[seq] - ql == 0 ? nullptr : to;
   }
   float S[DPT], P[DPT];
 #pragma unroll
   for (int i = 0; i < DPT; ++i) {
-    S[i] = (from && col_on && d0 + i < D) ? from[(int64_t)(d0 + i) * p.V] : 0.0f;
+    S[i] = (from && col_on && d0 + i < D) ? from[(d0 + i) * rs] : 0.0f;
     P[i] = 1.0f;
   }
   const float fixed = p.decay_kind == 1 ? p.decay[h] : 1.0f;
@@ -187,7 +194,7 @@ __global__ __launch_bounds__(1024) void matrix_scan_kernel(MatrixScanParams p, i
   if (to) {
 #pragma unroll
     for (int i = 0; i < DPT; ++i)
-      if (col_on && d0 + i < D) to[(int64_t)(d0 + i) * p.V] = S[i];
+      if (col_on && d0 + i < D) to[(d0 + i) * rs] = S[i];
   }
   if (p.a_out && chan && blockIdx.x == 0 && c == 0) {
 #pragma unroll
@@ -205,7 +212,7 @@ __global__ __launch_bounds__(256) void scan_carry_kernel(ScanCarryParams p) {
   const int64_t DV = (int64_t)p.D * p.V;
   const int n = p.s_count[seq];
   if (e >= DV || n <= 0 || p.q_len[seq] <= 0) return;
-  const int d = (int)(e / p.V);
+  const int d = p.V % kScanCols == 0 ? (int)((e / kScanCols) % p.D) : (int)(e / p.V);  // tile-major or plain entries
   const bool fresh = p.ctx_len[seq] - p.q_len[seq] == 0;
   float S = fresh ? 0.0f : p.state[((int64_t)p.state_slot[seq] * p.H + h) * DV + e];
   const float fixed = p.decay_kind == 1 ? p.decay[h] : 1.0f;

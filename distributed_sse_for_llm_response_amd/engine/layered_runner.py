@@ -274,24 +274,22 @@ class LayeredRunner(RunnerBase):
 
     # ------------------------------------------------------------------ pre-norm designs, matrix-state mixers
     def _prenorm_buffers(self, M: int) -> dict:
-        """Scratch of a step of M rows, each sized for the widest layer: `big` / `small` take the fused projections'
-        fp32 outputs (their column ranges are the mixer's q, k, v, gates), `cv` the convolution's, `z` the per-channel
+        """Scratch of a step of M rows, each sized for the widest layer: `big` takes the fused projection's fp32 output
+        (its column ranges are the mixer's q, k, v and gates), `cv` the convolution's, `z` the per-channel
         decays, `qa` the attention's normed and rotated queries, `o` the recurrences' outputs, `ao` a mixer's gated
         output in the element type (the output projection's input), `y2` the second mixer of a parallel pair."""
         cfg, dev = self.cfg, self.device
         f32 = dict(device=dev, dtype=torch.float32)
         el = dict(device=dev, dtype=self.dtype)
-        big = small = cv = z = qa = o = ff = 1
+        big = cv = z = qa = o = ff = 1
         for i, L in enumerate(cfg.layers):
             m = L.mixer
             if L.kind == "delta":
-                c = 2 * m.kv_heads * m.dim + m.heads * m.vdim
-                big, small, cv, o = max(big, c + m.heads * m.vdim), max(small, 2 * m.heads), max(cv, c), max(o, m.heads * m.vdim)
+                big, cv = max(big, self.w.layers[i].mix.n_big), max(cv, 2 * m.kv_heads * m.dim + m.heads * m.vdim)
+                o = max(o, m.heads * m.vdim)
             elif L.kind == "parallel":
                 a, r = m.left, m.right
-                nl = (a.heads + a.kv_heads) * a.dim + a.kv_heads * a.vdim
-                big = max(big, nl + 2 * r.heads * (r.dim + r.vdim))
-                small = max(small, a.heads + self.w.layers[i].mix.a2.shape[1])
+                big = max(big, self.w.layers[i].mix.n_big)
                 z, qa = max(z, r.heads * r.dim), max(qa, a.heads * a.dim)
                 o = max(o, a.heads * a.vdim, r.heads * r.vdim)
             else:
@@ -299,7 +297,7 @@ class LayeredRunner(RunnerBase):
             if L.mlp is not None:
                 ff = max(ff, L.mlp.ff)
         return {"y2": torch.zeros(M, cfg.width, **f32), "big": torch.zeros(M * big, **f32),
-                "small": torch.zeros(M * small, **f32), "cv": torch.zeros(M * cv, **f32), "z": torch.zeros(M * z, **f32),
+                "cv": torch.zeros(M * cv, **f32), "z": torch.zeros(M * z, **f32),
                 "qa": torch.zeros(M * qa, **f32), "o": torch.zeros(M * o, **f32), "ao": torch.zeros(M * o, **el),
                 "gu": torch.zeros(M * 2 * ff, **f32), "h": torch.zeros(M * ff, **el)}
 
@@ -357,7 +355,8 @@ class LayeredRunner(RunnerBase):
                 s_first, s_count, cm = g["ck"]
                 D = k.shape[2]
                 scr = self._scratch(d, "scan_s", cm.shape[1] * H * D * V)
-                ascr = self._scratch(d, "scan_a", cm.shape[1] * H * D) if decay is not None and decay.dim() == 3 else None
+                chan = decay is not None and decay.dim() == 3
+                ascr = self._scratch(d, "scan_a", cm.shape[1] * H * D) if chan else None
                 ops.matrix_scan_chunked(q, k, v, decay, self.state.state[ri], g["qs"], g["ql"], g["ctx"], g["ss"],
                                         s_first, s_count, cm, scr, ascr, o, q_scale)
             else:
@@ -370,11 +369,10 @@ class LayeredRunner(RunnerBase):
     def _delta(self, ri: int, m, Lw, M: int, d: dict, pos, slots, groups: list) -> None:
         H, G, D, V = m.heads, m.kv_heads, m.dim, m.vdim
         C = 2 * G * D + H * V
-        big = d["big"][:M * (C + H * V)].view(M, C + H * V)
-        small = d["small"][:M * 2 * H].view(M, 2 * H)
+        big = d["big"][:M * Lw.n_big].view(M, Lw.n_big)
+        small = big[:, C + H * V:C + H * V + 2 * H]   # per-head decay and write-strength pre-activations
         cv = d["cv"][:M * C].view(M, C)
         self._lin(d["xb"], Lw.big, Lw.big_t, big)
-        ops.gemm_rm(d["xb"], Lw.small, small)
         for g in groups:
             ops.conv_state(big[:, :C], Lw.conv, None, self.state.tail.get(ri), g["qs"], g["ql"], g["ctx"], g["ss"], cv,
                            None, None, 1)
@@ -383,8 +381,8 @@ class LayeredRunner(RunnerBase):
         ops.norm_rope_rows(k, None, pos, None, k, None, 2, UNIT_EPS, 1.0)
         ops.gate_math(small[:, :H], 0, Lw.a_log, Lw.dt_bias)
         ops.gate_math(small[:, H:], 1)
-        self._scan_out(ri, Lw.norm, big[:, C:], H, V, M, d, q, k, v, small[:, :H], small[:, H:], groups, 1.0, Lw.o,
-                       Lw.o_t, d["y"])
+        self._scan_out(ri, Lw.norm, big[:, C:C + H * V], H, V, M, d, q, k, v, small[:, :H], small[:, H:], groups, 1.0,
+                       Lw.o, Lw.o_t, d["y"])
 
     def _parallel(self, ri: int, m, Lw, M: int, d: dict, pos, slots, groups: list) -> None:
         a, r = m.left, m.right
@@ -392,15 +390,15 @@ class LayeredRunner(RunnerBase):
         Hr, Dr, Vr = r.heads, r.dim, r.vdim
         NL, NR = (H + G) * D + G * V, 2 * Hr * (Dr + Vr)
         rank = Lw.a2.shape[1]
-        big = d["big"][:M * (NL + NR)].view(M, NL + NR)
-        small = d["small"][:M * (H + rank)].view(M, H + rank)
+        big = d["big"][:M * Lw.n_big].view(M, Lw.n_big)
+        small = big[:, NL + NR:NL + NR + H + rank]    # the attention's per-head gates | the decay's inner projection
         self._lin(d["xb"], Lw.big, Lw.big_t, big)
-        ops.gemm_rm(d["xb"], Lw.small, small)
         # left: softmax attention with a sink over this run's pages
         rope = self._rope.get(a.rot)
         qa = d["qa"][:M * H * D].view(M, H, D)
         ops.norm_rope_rows(self._cols(big, 0, H, D), Lw.q_norm, pos, rope, qa, None, 1, self.cfg.eps, 1.0)
-        ops.norm_rope_rows(self._cols(big, H * D, G, D), Lw.k_norm, pos, rope, self.kv.k[ri], slots, 1, self.cfg.eps, 1.0)
+        ops.norm_rope_rows(self._cols(big, H * D, G, D), Lw.k_norm, pos, rope, self.kv.k[ri], slots, 1, self.cfg.eps,
+                           1.0)
         vt = self.kv.vt.get(ri)
         ops.norm_rope_rows(self._cols(big, (H + G) * D, G, V), None, pos, None, self.kv.v[ri], slots, 0, 0.0, 1.0, vt)
         ao = d["ao"][:M * H * V].view(M, H, V)
@@ -422,7 +420,7 @@ class LayeredRunner(RunnerBase):
         c0 = NL
         q, k = self._cols(big, c0, Hr, Dr), self._cols(big, c0 + Hr * Dr, Hr, Dr)
         v = self._cols(big, c0 + 2 * Hr * Dr, Hr, Vr)
-        gate = big[:, c0 + 2 * Hr * Dr + Hr * Vr:]
+        gate = big[:, c0 + 2 * Hr * Dr + Hr * Vr:NL + NR]
         self._scan_out(ri, Lw.rnorm, gate, Hr, Vr, M, d, q, k, v, z.view(M, Hr, Dr), None, groups, Dr ** -0.5, Lw.ro,
                        Lw.ro_t, d["y2"])
         ops.rms_mix(d["y"], Lw.left_out, d["y2"], Lw.right_out, self.cfg.eps, 0.5, d["y"])
@@ -499,7 +497,8 @@ class LayeredRunner(RunnerBase):
         """Packed metadata of prompt portions whose rows start at `row0`: one pinned upload.  Returns (T, q_start
         list, device dict: ids / pos / slots per row, qs / ql / ctx / ss per sequence, ws / wt work items, bt)."""
         n = len(seqs)
-        ids_l, pos_l, slots_l, qs, ql, ctx, ss, ws, wt, fs, ft, hs, ht = [], [], [], [], [], [], [], [], [], [], [], [], []
+        ids_l, pos_l, slots_l, qs, ql, ctx, ss = [], [], [], [], [], [], []
+        ws, wt, fs, ft, hs, ht = [], [], [], [], [], []
         bt = torch.zeros(n, self.max_blocks, dtype=torch.int32)
         row = 0
         for i, s in enumerate(seqs):
@@ -525,8 +524,8 @@ class LayeredRunner(RunnerBase):
             ht += list(range(nh))
             row += m
         T = row
-        meta = torch.from_numpy(np.concatenate(ids_l + pos_l + slots_l + [np.asarray(qs + ql + ctx + ss + ws + wt + fs + ft + hs + ht,
-                                                                                     dtype=np.int64)]).astype(np.int32))
+        lists = np.asarray(qs + ql + ctx + ss + ws + wt + fs + ft + hs + ht, dtype=np.int64)
+        meta = torch.from_numpy(np.concatenate(ids_l + pos_l + slots_l + [lists]).astype(np.int32))
         if self.device.type == "cuda":
             meta = meta.pin_memory().to(self.device, non_blocking=True)
             bt = bt.pin_memory().to(self.device, non_blocking=True)

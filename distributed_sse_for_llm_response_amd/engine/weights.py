@@ -369,9 +369,9 @@ def load_layered_dir(cfg, path: str, device="cpu", dtype=torch.bfloat16) -> Laye
 
 # ---------------------------------------------------------------------------------------------------------------------
 # Pre-norm designs with matrix-state mixers (models/surodra.py): every projection that reads the same input is ONE
-# weight (its outputs are column ranges of one fp32 GEMM output); the few-row projections (gates per head, the decay's
-# inner projection) are grouped into a second, small one so that the large one keeps an aligned row count.  Norm gains,
-# sinks and decay parameters are fp32 in both element types.
+# weight (its outputs are column ranges of one fp32 GEMM output) -- also the few-row ones (gates per head, the decay's
+# inner projection), which come last; zero rows pad the fused weight to a multiple of 128 rows when it is large enough
+# for the tiled-layout GEMMs.  Norm gains, sinks and decay parameters are fp32 in both element types.
 @dataclass
 class TanhNormWeights:
     alpha: torch.Tensor      # [1] fp32
@@ -381,8 +381,8 @@ class TanhNormWeights:
 
 @dataclass
 class DeltaWeights:
-    big: torch.Tensor        # rows [q (G D) | k (G D) | v (H V) | g (H V)] x W
-    small: torch.Tensor      # rows [a (H) | b (H)] x W
+    big: torch.Tensor        # rows [q (G D) | k (G D) | v (H V) | g (H V) | a (H) | b (H) | zero rows] x W
+    n_big: int               # rows of big (the width of its output)
     conv: torch.Tensor       # [2 G D + H V, taps] fp32: the taps of q | k | v
     a_log: torch.Tensor      # [H] fp32
     dt_bias: torch.Tensor    # [H] fp32
@@ -394,8 +394,8 @@ class DeltaWeights:
 
 @dataclass
 class ParallelWeights:
-    big: torch.Tensor        # rows [left q | left k | left v | right q | right k | right v | right g] x W
-    small: torch.Tensor      # rows [left g (H) | right a1 (rank)] x W
+    big: torch.Tensor        # rows [left q | k | v | right q | k | v | g | left g (H) | right a1 (rank) | zeros] x W
+    n_big: int
     q_norm: torch.Tensor     # fp32
     k_norm: torch.Tensor
     sink: torch.Tensor       # [H] fp32
@@ -455,7 +455,11 @@ def convert_surodra(cfg, tensors: dict, device="cpu", dtype=torch.bfloat16) -> L
         return tensors[name].to(device=device, dtype=torch.float32).contiguous()
 
     def cat(*names):
-        return torch.cat([t(n) for n in names], dim=0).contiguous()
+        """The named projections as one weight; large ones are padded with zero rows to a multiple of 128 rows."""
+        w = torch.cat([t(n) for n in names], dim=0)
+        if w.shape[0] >= TILED_MIN and w.shape[0] % 128:
+            w = torch.cat([w, w.new_zeros(128 - w.shape[0] % 128, w.shape[1])], dim=0)
+        return w.contiguous()
 
     def norm(name):
         return TanhNormWeights(alpha=f(name + ".alpha").reshape(1), w=f(name), b=f(name + ".b"))
@@ -464,7 +468,8 @@ def convert_surodra(cfg, tensors: dict, device="cpu", dtype=torch.bfloat16) -> L
     for i, L in enumerate(cfg.layers):
         p = f"l{i}.mix."
         if L.kind == "delta":
-            mix = DeltaWeights(big=cat(p + "q", p + "k", p + "v", p + "g"), small=cat(p + "a", p + "b"),
+            big = cat(p + "q", p + "k", p + "v", p + "g", p + "a", p + "b")
+            mix = DeltaWeights(big=big, n_big=big.shape[0],
                                conv=torch.cat([f(p + "q.conv"), f(p + "k.conv"), f(p + "v.conv")]).contiguous(),
                                a_log=f(p + "A_log"), dt_bias=f(p + "dt_bias"), norm=f(p + "norm"), o=t(p + "o"))
             _tile_fields(mix, ("big", "o"))
@@ -472,8 +477,8 @@ def convert_surodra(cfg, tensors: dict, device="cpu", dtype=torch.bfloat16) -> L
             l, r = p + "left.", p + "right."
             if tensors[r + "a2"].shape[1] != tensors[r + "a1"].shape[0]:
                 raise ValueError(f"layer {i}: the decay's two projections disagree on their inner width")
-            mix = ParallelWeights(big=cat(l + "q", l + "k", l + "v", r + "q", r + "k", r + "v", r + "g"),
-                                  small=cat(l + "g", r + "a1"), q_norm=f(l + "q.norm"), k_norm=f(l + "k.norm"),
+            big = cat(l + "q", l + "k", l + "v", r + "q", r + "k", r + "v", r + "g", l + "g", r + "a1")
+            mix = ParallelWeights(big=big, n_big=big.shape[0], q_norm=f(l + "q.norm"), k_norm=f(l + "k.norm"),
                                   sink=f(l + "sink"), a2=f(r + "a2"), a2_b=f(r + "a2.b"), rnorm=f(r + "norm"),
                                   lo=t(l + "o"), ro=t(r + "o"), left_out=f(l + "out"), right_out=f(r + "out"))
             _tile_fields(mix, ("big", "lo", "ro"))
@@ -495,7 +500,7 @@ def convert_surodra(cfg, tensors: dict, device="cpu", dtype=torch.bfloat16) -> L
 
 
 def load_surodra_dir(cfg, path: str, device="cpu", dtype=torch.bfloat16) -> LayeredWeights:
-    """``*.safetensors`` of a checkpoint directory -> the engine's layout (the loader executes nothing from the files)."""
+    """``*.safetensors`` of a checkpoint directory -> the engine's layout (the loader executes nothing from them)."""
     from pathlib import Path
 
     from safetensors.torch import load_file

@@ -213,6 +213,23 @@ def matrix_scan(q, k, v, decay, beta, state, q_start, q_len, ctx_len, state_slot
         lref.matrix_scan(q, k, v, decay, beta, state, q_start, q_len, ctx_len, state_slot, out, q_scale)
 
 
+def scan_state_plain(state):
+    """A GPU matrix state [slots, H, D, V] as the plain [.., D, V] matrices it stands for.  The scan kernels keep an
+    entry tile-major ([H][V / 16][D][16]) when V is a multiple of 16; CPU tensors are plain already."""
+    S, H, D, V = state.shape
+    if not state.is_cuda or V % 16:
+        return state
+    return state.view(S, H, V // 16, D, 16).permute(0, 1, 3, 2, 4).reshape(S, H, D, V)
+
+
+def scan_state_from_plain(plain):
+    """The inverse of scan_state_plain for a GPU tensor: plain matrices -> the kernels' layout."""
+    S, H, D, V = plain.shape
+    if not plain.is_cuda or V % 16:
+        return plain
+    return plain.view(S, H, D, V // 16, 16).permute(0, 1, 3, 2, 4).reshape(S, H, D, V).contiguous()
+
+
 SCAN_CHUNK = 64        # tokens per chunk of the two-level walk
 SCAN_CHUNKED_FROM = 256  # rows of a prompt group from which matrix_scan_chunked pays
 

@@ -231,11 +231,13 @@ def test_matrix_scan(H, G, D, V, mode):
     qg = wg[:, 2:2 + G * D].unflatten(1, (G, D))
     kg = wg[:, 2 + G * D:2 + 2 * G * D].unflatten(1, (G, D))
     vg = wg[:, 2 + 2 * G * D:2 + 2 * G * D + H * V].unflatten(1, (H, V))
-    st, o = c(state0.clone()), torch.zeros(T, H, V, device=dev())
+    from distributed_sse_for_llm_response_amd.ops.layers import scan_state_from_plain, scan_state_plain
+
+    st, o = scan_state_from_plain(c(state0.clone())), torch.zeros(T, H, V, device=dev())
     ops.matrix_scan(qg, kg, vg, c(decay), c(beta), st, c(qs), c(i32(ql)), c(i32(ctx)), c(i32(slot)), o, 0.3)
     close(o, o_ref, 2e-5)
-    close(st, st_ref, 2e-5)
-    assert torch.equal(st[3].cpu(), state0[3])   # the inactive sequence's slot is untouched
+    close(scan_state_plain(st), st_ref, 2e-5)
+    assert torch.equal(scan_state_plain(st)[3].cpu(), state0[3])   # the inactive sequence's slot is untouched
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -290,7 +292,7 @@ def test_matrix_scan_two_level_walk(H, G, D, V, mode):
     """Long portions walked in chunks (parallel from zeros, carry, parallel again) against the plain reference walk:
     a fresh prompt that ends inside a chunk, a later portion continued from its slot, one exactly one chunk long, one
     shorter than a chunk."""
-    from distributed_sse_for_llm_response_amd.ops.layers import scan_chunks
+    from distributed_sse_for_llm_response_amd.ops.layers import scan_chunks, scan_state_from_plain, scan_state_plain
 
     g = torch.Generator().manual_seed(11)
     ql, ctx, slot = [200, 131, 64, 5], [200, 300, 64, 90], [2, 0, 3, 1]
@@ -307,11 +309,11 @@ def test_matrix_scan_two_level_walk(H, G, D, V, mode):
     s_first, s_count, rows = scan_chunks(qs, ql, slot)
     assert s_count == [4, 3, 1, 1]
     c = lambda t: None if t is None else t.to(dev())  # noqa: E731
-    st, o = c(state0.clone()), torch.zeros(T, H, V, device=dev())
+    st, o = scan_state_from_plain(c(state0.clone())), torch.zeros(T, H, V, device=dev())
     n = len(rows[0])
     scr = torch.full((n * H * D * V,), float("nan"), device=dev())
     ascr = torch.full((n * H * D,), float("nan"), device=dev()) if mode == "channel" else None
     ops.matrix_scan_chunked(c(q), c(k), c(v), c(decay), st, c(i32(qs)), c(i32(ql)), c(i32(ctx)), c(i32(slot)),
                             c(i32(s_first)), c(i32(s_count)), c(i32(rows)), scr, ascr, o, 0.5)
     close(o, o_ref, 3e-5)
-    close(st, st_ref, 3e-5)
+    close(scan_state_plain(st), st_ref, 3e-5)
