@@ -84,6 +84,7 @@ struct MatrixScanParams {
   const float* src;
   float* dst;
   int no_out;            // 1: a pass that only produces end states
+  int portions;          // 1: the rows are prompt portions (many rows per sequence): the wave-local kernel
   float* a_out;          // [nseq, H, D] product of the chunk's per-channel decays (decay_kind 3) or null
 };
 

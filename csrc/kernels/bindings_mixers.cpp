@@ -301,6 +301,7 @@ void matrix_scan(const Tensor& q, const Tensor& k, const Tensor& v, const OptTen
   p.state_slot = state_slot.data_ptr<int>();
   p.out = out.data_ptr<float>();
   p.q_scale = (float)q_scale;
+  p.portions = T > 2 * p.nseq;  // more than a row or two per sequence: prompt portions, not a decode step
   DSSE_CHECK_HIP(dsse_matrix_scan(&p, cur_stream()));
 }
 
@@ -370,6 +371,7 @@ void matrix_scan_chunked(const Tensor& q, const Tensor& k, const Tensor& v, cons
   p.state_slot = cm + 5 * N;
   p.out = out.data_ptr<float>();
   p.q_scale = (float)q_scale;
+  p.portions = 1;
   // pass 1: from zeros, end states into scratch
   p.q_len = cm + 2 * N;
   p.src_idx = cm + 3 * N, p.dst_idx = cm + 4 * N;

@@ -203,6 +203,197 @@ __global__ __launch_bounds__(1024) void matrix_scan_kernel(MatrixScanParams p, i
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// Prompt portions: the same recurrence with every sum over D INSIDE a wave.  A wave owns 4 columns of one (sequence,
+// head) and all D rows of them: lane (c, dg) holds rows dg DPT + i of column c (16 lane groups, DPT = D / 16 rounded
+// up to a power of two), a dot product over D is DPT FMAs per lane, two row rotations inside each 16-lane row and
+// two row swaps -- no LDS, no barrier, also for the delta rule.  The four waves of a workgroup own 16 adjacent columns
+// (one tile of the state entry) and share the head's staged k, q and decays; the only workgroup barrier is per token
+// block.  With rows spread this thin the chain per token is short enough that the walk is no longer dominated by the
+// delta rule's cross-wave sum; the state is touched in 16-byte pieces, which a prompt portion does once.
+template <int CTRL>
+DEV float dpp_rot(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+// sum over the 16 lane groups of a wave (lanes with the same lane & 3): quads of a 16-lane row, then the four rows
+DEV float groups16_sum(float v) {
+  v += dpp_rot<0x128>(v);  // row_ror:8
+  v += dpp_rot<0x124>(v);  // row_ror:4
+  return rows4_sum(v);
+}
+
+template <int DPT>
+DEV float dot_dpt(const float* S, const float* x) {
+  if constexpr (DPT >= 4) {
+    float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < DPT; i += 2) {
+      a0 += S[i] * x[i];
+      a1 += S[i + 1] * x[i + 1];
+    }
+    return a0 + a1;
+  } else {
+    float a = 0.f;
+#pragma unroll
+    for (int i = 0; i < DPT; ++i) a += S[i] * x[i];
+    return a;
+  }
+}
+
+template <int DPT, int TB, bool DELTA>
+__global__ __launch_bounds__(256) void matrix_scan_wave_kernel(MatrixScanParams p) {
+  constexpr int Dp = 16 * DPT;       // rows of S a wave holds (>= D; rows past D stay zero)
+  constexpr int E = TB * Dp / 256;   // staged elements of k (and q, a) per thread and block
+  static_assert(E >= 1 && E * 256 == TB * Dp, "a block's staging divides evenly over the workgroup");
+  extern __shared__ __align__(16) float lds[];
+  const int seq = blockIdx.z, h = blockIdx.y;
+  const int ql = p.q_len[seq];
+  if (ql <= 0) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 3, dg = lane >> 2;
+  const int j = blockIdx.x * kScanCols + 4 * wave + c;
+  const bool col_on = j < p.V;
+  const int g = h / (p.H / p.G);
+  const int D = p.D;
+  const int d0 = dg * DPT;
+  const bool chan = p.decay_kind == 3;
+  // LDS: k[2][TB][Dp] | q[2][TB][Dp] | (a[2][TB][Dp]) | sc[2][2][TB] (beta, scalar decay)
+  float* ks = lds;
+  float* qs = ks + 2 * TB * Dp;
+  float* as = qs + 2 * TB * Dp;
+  float* sc = as + (chan ? 2 * TB * Dp : 0);
+  const int row0 = p.q_start[seq];
+  const bool tiled = p.V % kScanCols == 0;  // the state entry's layout: see matrix_scan_kernel
+  const int64_t rs = tiled ? kScanCols : p.V;
+  const int64_t col_off = tiled ? (int64_t)blockIdx.x * D * kScanCols + 4 * wave + c : j;
+  const int64_t entry = (int64_t)p.H * D * p.V;
+  const float* from;
+  float* to;
+  if (p.src_idx) {
+    const int si = p.src_idx[seq], di = p.dst_idx[seq];
+    from = si >= 0 ? p.src + si * entry + (int64_t)h * D * p.V + col_off : nullptr;
+    to = di >= 0 ? p.dst + di * entry + (int64_t)h * D * p.V + col_off : nullptr;
+  } else {
+    to = p.state + p.state_slot[seq] * entry + (int64_t)h * D * p.V + col_off;
+    from = p.ctx_len[seq] - ql == 0 ? nullptr : to;
+  }
+  float S[DPT], P[DPT];
+#pragma unroll
+  for (int i = 0; i < DPT; ++i) {
+    S[i] = (from && col_on && d0 + i < D) ? from[(d0 + i) * rs] : 0.0f;
+    P[i] = 1.0f;
+  }
+  const float fixed = p.decay_kind == 1 ? p.decay[h] : 1.0f;
+  float nk[E], nq[E], na[E], nv[TB], nsc0 = 0.f, nsc1 = fixed;
+  auto request = [&](int b) {  // block b (tokens [b TB, b TB + TB)) into registers
+    const int t0 = b * TB;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int idx = e * 256 + tid;
+      const int t = idx / Dp, d = idx % Dp;
+      const bool on = t0 + t < ql && d < D;  // padded channels and tokens past the end are staged as k = q = 0, a = 1
+      const int64_t row = row0 + t0 + t;
+      nk[e] = on ? p.k[row * p.ldk + g * D + d] : 0.0f;
+      nq[e] = on ? p.q[row * p.ldq + g * D + d] * p.q_scale : 0.0f;
+      na[e] = (on && chan) ? p.decay[row * p.ldd + h * D + d] : 1.0f;
+    }
+#pragma unroll
+    for (int t = 0; t < TB; ++t)
+      nv[t] = (col_on && t0 + t < ql) ? p.v[(int64_t)(row0 + t0 + t) * p.ldv + h * p.V + j] : 0.0f;
+    if (tid < TB && t0 + tid < ql) {
+      const int64_t row = row0 + t0 + tid;
+      if (DELTA) nsc0 = p.beta[row * p.ldb + h];
+      if (p.decay_kind == 2) nsc1 = p.decay[row * p.ldd + h];
+    }
+  };
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int idx = e * 256 + tid;
+      ks[buf * TB * Dp + idx] = nk[e];
+      qs[buf * TB * Dp + idx] = nq[e];
+      if (chan) as[buf * TB * Dp + idx] = na[e];
+    }
+    if (tid < TB) {
+      sc[(buf * 2 + 0) * TB + tid] = nsc0;
+      sc[(buf * 2 + 1) * TB + tid] = nsc1;
+    }
+  };
+  auto token = [&](int buf, int t, float v) -> float {  // updates S, returns the column's read-out (in all its lanes)
+    const float* kb = ks + (buf * TB + t) * Dp + d0;
+    const float* qb = qs + (buf * TB + t) * Dp + d0;
+    if (chan) {
+      const float* ab = as + (buf * TB + t) * Dp + d0;
+#pragma unroll
+      for (int i = 0; i < DPT; ++i) S[i] *= ab[i];
+      if (p.a_out) {  // uniform: the chunk's decay product for the carry
+#pragma unroll
+        for (int i = 0; i < DPT; ++i) P[i] *= ab[i];
+      }
+    } else if (p.decay_kind != 0) {
+      const float sa = sc[(buf * 2 + 1) * TB + t];
+#pragma unroll
+      for (int i = 0; i < DPT; ++i) S[i] *= sa;
+    }
+    float u = v;
+    if (DELTA) u = sc[(buf * 2 + 0) * TB + t] * (v - groups16_sum(dot_dpt<DPT>(S, kb)));
+#pragma unroll
+    for (int i = 0; i < DPT; ++i) S[i] += kb[i] * u;
+    return groups16_sum(dot_dpt<DPT>(S, qb));
+  };
+  const int nblocks = (ql + TB - 1) / TB;
+  request(0);
+  stage(0);
+  const bool writer = dg == 0 && col_on && !p.no_out;
+  for (int b = 0; b < nblocks; ++b) {
+    const int buf = b & 1;
+    float cv[TB];
+#pragma unroll
+    for (int t = 0; t < TB; ++t) cv[t] = nv[t];
+    if (b + 1 < nblocks) request(b + 1);  // in flight while this block is walked
+    lds_barrier();                        // this block's staging is visible; the other buffer has been read
+    float* out = p.out + ((int64_t)(row0 + b * TB) * p.H + h) * p.V + j;
+    if (ql - b * TB >= TB) {  // a full block: no branches between its tokens
+#pragma unroll
+      for (int t = 0; t < TB; ++t) {
+        const float o = token(buf, t, cv[t]);
+        if (writer) out[(int64_t)t * p.H * p.V] = o;
+      }
+    } else {
+      const int nt = ql - b * TB;
+#pragma unroll
+      for (int t = 0; t < TB; ++t) {
+        if (t < nt) {  // uniform
+          const float o = token(buf, t, cv[t]);
+          if (writer) out[(int64_t)t * p.H * p.V] = o;
+        }
+      }
+    }
+    if (b + 1 < nblocks) stage(buf ^ 1);  // that buffer was last read in block b - 1, before this block's barrier
+  }
+  if (to) {
+#pragma unroll
+    for (int i = 0; i < DPT; ++i)
+      if (col_on && d0 + i < D) to[(d0 + i) * rs] = S[i];
+  }
+  if (p.a_out && chan && blockIdx.x == 0 && wave == 0 && c == 0) {
+#pragma unroll
+    for (int i = 0; i < DPT; ++i)
+      if (d0 + i < D) p.a_out[((int64_t)seq * p.H + h) * D + d0 + i] = P[i];
+  }
+}
+
+template <int DPT, int TB>
+hipError_t launch_wave(const MatrixScanParams& p, hipStream_t st) {
+  constexpr int Dp = 16 * DPT;
+  dim3 grid((p.V + kScanCols - 1) / kScanCols, p.H, p.nseq);
+  const size_t lds = (size_t)((p.decay_kind == 3 ? 6 : 4) * TB * Dp + 4 * TB) * sizeof(float);
+  if (lds > 64 * 1024 || p.D > Dp) return hipErrorInvalidValue;
+  if (p.beta) hipLaunchKernelGGL((matrix_scan_wave_kernel<DPT, TB, true>), grid, dim3(256), lds, st, p);
+  else hipLaunchKernelGGL((matrix_scan_wave_kernel<DPT, TB, false>), grid, dim3(256), lds, st, p);
+  return hipGetLastError();
+}
+
 // S_in of every chunk of a sequence: S_in[0] = the slot's state (zeros at position 0), S_in[c + 1] = A_c S_in[c] + B_c
 // with B_c the chunk's end state from zeros (found in its scratch entry, which then receives S_in[c]) and A_c the
 // product of its decays.  One thread per state element; a sequence has a handful of chunks.
@@ -252,6 +443,14 @@ hipError_t launch(const MatrixScanParams& p, hipStream_t st) {
 extern "C" hipError_t dsse_matrix_scan(const dsse::MatrixScanParams* p, hipStream_t st) {
   if (p->nseq <= 0 || p->H <= 0) return hipSuccess;
   if (p->D < 1 || p->D > 512 || p->V < 1 || p->G < 1 || p->H % p->G) return hipErrorInvalidValue;
+  if (p->portions) {  // prompt portions: all sums inside a wave (rows per lane = D / 16 rounded up to a power of two)
+    if (p->D <= 16) return dsse::launch_wave<1, 16>(*p, st);
+    if (p->D <= 32) return dsse::launch_wave<2, 16>(*p, st);
+    if (p->D <= 64) return dsse::launch_wave<4, 16>(*p, st);
+    if (p->D <= 128) return dsse::launch_wave<8, 16>(*p, st);
+    if (p->D <= 256) return dsse::launch_wave<16, 8>(*p, st);
+    return dsse::launch_wave<32, 4>(*p, st);
+  }
   // rows of S per lane (a wave holds 4 DPT rows of 16 columns, a workgroup up to 16 waves) and tokens per block (as
   // long as 64 KB of LDS allow)
   if (p->D <= 64) return dsse::launch<2, 16>(*p, st);

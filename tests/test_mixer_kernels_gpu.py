@@ -317,3 +317,29 @@ def test_matrix_scan_two_level_walk(H, G, D, V, mode):
                             c(i32(s_first)), c(i32(s_count)), c(i32(rows)), scr, ascr, o, 0.5)
     close(o, o_ref, 3e-5)
     close(scan_state_plain(st), st_ref, 3e-5)
+
+
+@pytest.mark.parametrize("H,G,D,V", [(4, 2, 32, 32), (2, 1, 128, 64), (1, 1, 300, 70)])
+@pytest.mark.parametrize("mode", ["delta", "channel", "fixed"])
+def test_matrix_scan_decode_rows(H, G, D, V, mode):
+    """One row per sequence (a decode step: the kernel that keeps the state traffic coalesced), one slot inactive,
+    one sequence at position 0."""
+    from distributed_sse_for_llm_response_amd.ops.layers import scan_state_from_plain, scan_state_plain
+
+    g = torch.Generator().manual_seed(12)
+    ql, ctx, slot = [1, 1, 0, 1, 1], [9, 1, 4, 300, 2], [4, 0, 3, 1, 2]
+    qs = i32([0, 1, 2, 3, 4])
+    T = 5
+    q, k = torch.randn(T, G, D, generator=g) * 0.3, torch.randn(T, G, D, generator=g) * 0.3
+    v = torch.randn(T, H, V, generator=g)
+    decay = {"delta": torch.rand(T, H, generator=g) * 0.5 + 0.5, "channel": torch.rand(T, H, D, generator=g) * 0.3 + 0.7,
+             "fixed": torch.linspace(0.5, 0.99, H)}[mode]
+    beta = torch.rand(T, H, generator=g) if mode == "delta" else None
+    state0 = torch.randn(5, H, D, V, generator=g)
+    st_ref, o_ref = state0.clone(), torch.zeros(T, H, V)
+    lref.matrix_scan(q, k, v, decay, beta, st_ref, qs, i32(ql), i32(ctx), i32(slot), o_ref, 0.7)
+    c = lambda t: None if t is None else t.to(dev())  # noqa: E731
+    st, o = scan_state_from_plain(c(state0.clone())), torch.zeros(T, H, V, device=dev())
+    ops.matrix_scan(c(q), c(k), c(v), c(decay), c(beta), st, c(qs), c(i32(ql)), c(i32(ctx)), c(i32(slot)), o, 0.7)
+    close(o, o_ref, 2e-5)
+    close(scan_state_plain(st), st_ref, 2e-5)
