@@ -8,19 +8,22 @@
 //     S = S + k u^T
 //     o = S^T (q_scale q)           the read-out sees the current token's write
 //
+// Two kernels: this one for decode-sized steps (a row or two per sequence: what counts is the state traffic) and the
+// wave-local one further down for prompt portions (what counts is the chain per token).
+//
 // Column j of S evolves independently of the other columns, so the work is laid out by columns: a workgroup owns 16
 // columns of one (sequence, head).  Lane (c, dg) of wave r holds DPT rows of column c -- rows (4 r + dg) DPT + i -- in
 // registers, so a dot product over D is DPT FMAs per lane, a sum over the wave's four 16-lane rows (two row swaps, no
-// LDS) and a short sum over the waves through LDS.  A small DPT spreads one head's state over many waves: what bounds a
-// prompt portion is the dependent chain per token, and it is shortest when every lane holds few rows.
+// LDS) and a short sum over the waves through LDS.  A small DPT spreads one head's state over many waves, so a decode
+// step's pass over the state (read, update, write) is wide; a state entry is kept tile-major (below) so that the pass
+// moves whole lines.
 //
-// Tokens are taken in blocks of TB.  A block's k, q (and per-channel decays) are staged in LDS by the whole workgroup
-// with coalesced loads, and the NEXT block is already in flight (in registers) while the current one is walked.  The
-// read-out's partial sums of a whole block are reduced at the block's end, and a full block is walked without
-// branches, so without the delta rule the tokens of a block overlap (only S itself chains them); the delta rule needs
-// one workgroup barrier per token (its S^T k sum crosses the waves).  A decode step is one block of one token: one pass
-// over the state (read, update, write).  A sequence whose step starts at position 0 starts from S = 0; nothing is
-// cleared when a slot changes hands.
+// Tokens are taken in blocks of TB (a decode step is one block of one token; a step with two or three rows per
+// sequence walks them here too).  A block's k, q (and per-channel decays) are staged in LDS by the whole workgroup with
+// coalesced loads, the NEXT block is already in flight (in registers) while the current one is walked, the read-out's
+// partial sums of a block are reduced at the block's end, and the delta rule needs one workgroup barrier per token
+// (its S^T k sum crosses the waves).  A sequence whose step starts at position 0 starts from S = 0; nothing is cleared
+// when a slot changes hands.
 #include "api_mixers.h"
 
 namespace dsse {
@@ -68,22 +71,11 @@ __global__ __launch_bounds__(1024) void matrix_scan_kernel(MatrixScanParams p, i
   const int64_t rs = tiled ? kScanCols : p.V;  // floats between two rows of this lane's column
   const int64_t col_off = tiled ? (int64_t)blockIdx.x * D * kScanCols + c : j;
   const int64_t entry = (int64_t)p.H * D * p.V;
-  const float* from;
-  float* to;
-  if (p.src_idx) {
-    const int si = p.src_idx[seq], di = p.dst_idx[seq];
-    from = si >= 0 ? p.src + si * entry + (int64_t)h * D * p.V + col_off : nullptr;
-    to = di >= 0 ? p.dst + di * entry + (int64_t)h * D * p.V + col_off : nullptr;
-  } else {
-    to = p.state + p.state_slot[seq] * entry + (int64_t)h * D * p.V + col_off;
-    from = p.ctx_len[seq] - ql == 0 ? nullptr : to;
-  }
-  float S[DPT], P[DPT];
+  float* to = p.state + p.state_slot[seq] * entry + (int64_t)h * D * p.V + col_off;
+  const float* from = p.ctx_len[seq] - ql == 0 ? nullptr : to;  // a sequence's first step starts from zeros
+  float S[DPT];
 #pragma unroll
-  for (int i = 0; i < DPT; ++i) {
-    S[i] = (from && col_on && d0 + i < D) ? from[(d0 + i) * rs] : 0.0f;
-    P[i] = 1.0f;
-  }
+  for (int i = 0; i < DPT; ++i) S[i] = (from && col_on && d0 + i < D) ? from[(d0 + i) * rs] : 0.0f;
   const float fixed = p.decay_kind == 1 ? p.decay[h] : 1.0f;
   float nk[E], nq[E], na[E], nv[TB], nsc0 = 0.f, nsc1 = fixed;
   auto request = [&](int b) {  // block b (tokens [b TB, b TB + TB)) into registers
@@ -128,10 +120,6 @@ __global__ __launch_bounds__(1024) void matrix_scan_kernel(MatrixScanParams p, i
       const float* ab = as + (buf * TB + t) * Dp + d0;
 #pragma unroll
       for (int i = 0; i < DPT; ++i) S[i] *= ab[i];
-      if (p.a_out) {  // uniform: the chunk's decay product for the carry
-#pragma unroll
-        for (int i = 0; i < DPT; ++i) P[i] *= ab[i];
-      }
     } else if (p.decay_kind != 0) {
       const float sa = sc[(buf * 2 + 1) * TB + t];
 #pragma unroll
@@ -182,7 +170,7 @@ __global__ __launch_bounds__(1024) void matrix_scan_kernel(MatrixScanParams p, i
     }
     lds_barrier();  // the block's partial read-outs are complete; its staged inputs have been read
     // the block's [nt][16] outputs, one per thread
-    for (int idx = tid; idx < (p.no_out ? 0 : nt * kScanCols); idx += nthreads) {
+    for (int idx = tid; idx < nt * kScanCols; idx += nthreads) {
       const int t = idx / kScanCols, cc = idx % kScanCols;
       float o = 0.f;
       for (int w = 0; w < R; ++w) o += opart[(t * R + w) * kScanCols + cc];
@@ -191,16 +179,9 @@ __global__ __launch_bounds__(1024) void matrix_scan_kernel(MatrixScanParams p, i
     }
     if (b + 1 < nblocks) stage(buf ^ 1);
   }
-  if (to) {
 #pragma unroll
-    for (int i = 0; i < DPT; ++i)
-      if (col_on && d0 + i < D) to[(d0 + i) * rs] = S[i];
-  }
-  if (p.a_out && chan && blockIdx.x == 0 && c == 0) {
-#pragma unroll
-    for (int i = 0; i < DPT; ++i)
-      if (d0 + i < D) p.a_out[((int64_t)seq * p.H + h) * D + d0 + i] = P[i];
-  }
+  for (int i = 0; i < DPT; ++i)
+    if (col_on && d0 + i < D) to[(d0 + i) * rs] = S[i];
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
@@ -443,7 +424,7 @@ hipError_t launch(const MatrixScanParams& p, hipStream_t st) {
 extern "C" hipError_t dsse_matrix_scan(const dsse::MatrixScanParams* p, hipStream_t st) {
   if (p->nseq <= 0 || p->H <= 0) return hipSuccess;
   if (p->D < 1 || p->D > 512 || p->V < 1 || p->G < 1 || p->H % p->G) return hipErrorInvalidValue;
-  if (p->portions) {  // prompt portions: all sums inside a wave (rows per lane = D / 16 rounded up to a power of two)
+  if (p->portions || p->src_idx) {  // prompt portions (and every pass of the two-level walk): all sums inside a wave (rows per lane = D / 16 rounded up to a power of two)
     if (p->D <= 16) return dsse::launch_wave<1, 16>(*p, st);
     if (p->D <= 32) return dsse::launch_wave<2, 16>(*p, st);
     if (p->D <= 64) return dsse::launch_wave<4, 16>(*p, st);
