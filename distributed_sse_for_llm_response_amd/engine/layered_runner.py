@@ -1,4 +1,6 @@
-"""Forward passes of configuration-driven designs (models/muderax.py) on the layer-mechanism kernels (ops/layers.py).
+"""Forward passes of configuration-driven designs (models/muderax.py, models/surodra.py) on the layer-mechanism kernels
+(ops/layers.py).  Two block styles share the runner: sandwich norms on a sublayer's output (Muderax, described first)
+and pre-norm blocks around matrix-state mixers (Surodra, described after it).
 
 A step is a set of packed rows -- the B decode slots first (one row each, state on the device as in ModelRunner), then
 the rows of prompt portions -- that walk the layer list once:
@@ -16,9 +18,29 @@ the rows of prompt portions -- that walk the layer list once:
     after each sublayer     scalar_norm: stream += out / rms(out) * g; xb = rounding
     head                    scalar_norm (final) on the rows that need logits -> GEMM (fp32 logits)
 
+The pre-norm walk (`_prenorm_layers`) goes over layer RUNS -- a looped span of layers runs several times with the
+same weights and its own pages and state slots per pass:
+
+    stream_step             resid += m * (finished sublayer) (+ embedding again + the pass's vector at a pass's start);
+                            xb = tanh(alpha resid) w + b -- the add, the pass additions and the next norm in one kernel
+    delta layer             ONE fused GEMM [q | k | v | g | a | b] (fp32 out) -> conv_state over q | k | v (SiLU; slot
+                            tail) -> unit q, k per head -> gate_math (decay, write strength) -> matrix_scan (delta rule;
+                            slot state) -> gated_head_norm -> output GEMM
+    parallel layer          ONE fused GEMM for both halves -> left: norm_rope_rows (whole-row RMS norm + rotation: q to
+                            a buffer, k and v into this run's pages) -> sink_attention (MFMA form over transposed value
+                            pages for prompt portions and decode rows, row form otherwise) -> output GEMM; right: decay
+                            GEMM (fp32) -> gate_math -> matrix_scan (per-channel decay) -> gated_head_norm -> output
+                            GEMM; rms_mix of the two
+    retention layer         fused GEMM -> rotation of q, k -> matrix_scan (fixed decay) -> gated_head_norm -> output GEMM
+    feed-forward            fused [gate | up] GEMM -> gated_act (gelu) -> down GEMM
+    head                    stream_step (last add + final norm) -> head GEMM -> logit_cap (scale, tanh cap)
+
+Long prompt groups walk the recurrences without the delta rule in two levels (matrix_scan_chunked).
+
 The residual stream, norms, scores, router and recurrence are fp32 in both element types; ``dtype=torch.float32`` runs
 the projections in true fp32 as well (the exact mode).  The cache is paged with the engine's block tables and
-allocator (LatentKVCache); recurrent layers keep their state in the sequence's decode slot (RecurrentStateCache), so
+allocator (LatentKVCache, PagedKVCache); recurrent layers keep their state in the sequence's decode slot
+(RecurrentStateCache, MatrixStateCache), so
 slots and pages are handed from one sequence to the next with no clearing pass.  The decode step of each batch bucket
 is captured into a graph like ModelRunner's; prompt portions and mixed steps run eagerly.
 """
